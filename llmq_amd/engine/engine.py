@@ -23,10 +23,12 @@ import torch
 
 from llmq_amd import ops
 from llmq_amd.engine.config import EngineConfig
-from llmq_amd.engine.kv_cache import BlockAllocator, KVCache
+from llmq_amd.engine.kv_cache import (
+    BlockAllocator, KVCache, RecurrentStateCache, SlotAllocator,
+)
 from llmq_amd.engine.model_runner import ModelRunner
 from llmq_amd.engine.model_specs import ModelSpec, resolve_spec
-from llmq_amd.engine.models.llama import CausalLM
+from llmq_amd.engine.models import model_class_for
 from llmq_amd.engine.sampling_params import SamplingParams
 from llmq_amd.engine.scheduler import Scheduler, Sequence
 from llmq_amd.engine.tokenizer import load_tokenizer
@@ -97,9 +99,17 @@ class LLMEngine:
         tp = tp_size if tp_size is not None else config.tensor_parallel_size
         self.tp_size = tp
         self.tp_rank = tp_rank
-        if self.device.type == "cuda" and not ops.has_hip_ext():
+        model_cls = model_class_for(self.spec)
+        # HIP libraries the family's forward runs on ("main" unless the model
+        # class names others); the sampler's library loads at first sampling.
+        ext_groups = getattr(model_cls, "ext_groups", ("main",))
+        if self.device.type == "cuda":
             # Fail loudly: GPU execution must run the CDNA4 kernels.
-            ops._use_hip(torch.empty(1, device=self.device))
+            probe = torch.empty(1, device=self.device)
+            if "main" in ext_groups and not ops.has_hip_ext():
+                ops._use_hip(probe)
+            if "hybrid" in ext_groups and not ops.has_hybrid_ext():
+                ops._use_hybrid(probe)
         if self.device.type == "cuda":
             _enable_tuned_gemms()
         self.max_model_len = min(
@@ -111,14 +121,29 @@ class LLMEngine:
             self.spec.name, self.spec.family, self.spec.param_count() / 1e9,
             self.device, self.dtype, tp,
         )
-        self.model = CausalLM(self.spec, self.device, self.dtype, tp_rank, tp)
+        self.model = model_cls(self.spec, self.device, self.dtype, tp_rank, tp)
         self._load_or_init_weights()
         self.tokenizer = load_tokenizer(
             config.model, self.spec.vocab_size, self.spec.bos_token_id, self.spec.eos_token_id
         )
         self.kv_dtype = config.resolve_kv_dtype(self.device)
-        if self.kv_dtype == torch.float8_e4m3fn and self.spec.head_dim not in (128, 256):
-            raise ValueError("fp8 KV cache requires head_dim 128 or 256 (MFMA decode path)")
+        # Per-layer cache layout: uniform families derive it from the spec;
+        # a model class with layers of different shapes (or without keys)
+        # names its own, plus the shapes of its recurrent state.
+        if hasattr(self.model, "kv_layout"):
+            self.kv_layout = self.model.kv_layout()
+            if self.kv_dtype == torch.float8_e4m3fn:
+                raise ValueError("fp8 KV cache is not available for this model family")
+        else:
+            self.kv_layout = [
+                (self.spec.num_kv_heads // tp, self.spec.head_dim, self.spec.head_dim)
+            ] * self.spec.num_layers
+            if self.kv_dtype == torch.float8_e4m3fn and self.spec.head_dim not in (128, 256):
+                raise ValueError("fp8 KV cache requires head_dim 128 or 256 (MFMA decode path)")
+        state_layout = (
+            self.model.state_layout() if hasattr(self.model, "state_layout") else []
+        )
+        self.state_cache = RecurrentStateCache(state_layout, config.max_num_seqs, self.device)
         num_blocks = self._size_kv_cache()
         if tp > 1:
             # Deterministic lockstep requires an IDENTICAL KV pool on every
@@ -134,18 +159,22 @@ class LLMEngine:
                     num_blocks, synced,
                 )
             num_blocks = synced
-        kv_heads_local = self.spec.num_kv_heads // tp
         self.kv_cache = KVCache(
-            self.spec.num_layers, num_blocks, kv_heads_local,
-            config.kv_block_size, self.spec.head_dim, self.device, self.kv_dtype,
+            len(self.kv_layout), num_blocks, 0, config.kv_block_size, 0,
+            self.device, self.kv_dtype, layout=self.kv_layout,
         )
+        self.kv_cache.recurrent = self.state_cache
         self.allocator = BlockAllocator(num_blocks)
+        self.slot_allocator = (
+            SlotAllocator(config.max_num_seqs) if self.state_cache.active else None
+        )
         self.scheduler = Scheduler(
             self.allocator,
             config.kv_block_size,
             config.max_num_seqs,
             config.max_prefill_tokens,
             self.max_model_len,
+            slot_allocator=self.slot_allocator,
         )
         self.runner = ModelRunner(
             self.model, self.kv_cache, config, self.device, self.max_model_len
@@ -207,9 +236,8 @@ class LLMEngine:
         logger.info(
             "engine ready: %d KV blocks (%d tokens, %.1f GB), max_num_seqs=%d, graphs=%s",
             num_blocks, num_blocks * config.kv_block_size,
-            num_blocks * KVCache.block_bytes(
-                self.spec.num_layers, kv_heads_local, config.kv_block_size,
-                self.spec.head_dim, self.kv_dtype,
+            num_blocks * KVCache.layout_block_bytes(
+                self.kv_layout, config.kv_block_size, self.kv_dtype,
             ) / 2 ** 30 * 1.0,
             config.max_num_seqs,
             self.runner.use_graphs,
@@ -230,7 +258,6 @@ class LLMEngine:
 
     def _size_kv_cache(self) -> int:
         cfg = self.config
-        kv_heads_local = self.spec.num_kv_heads // self.tp_size
         if cfg.num_kv_blocks is not None:
             return cfg.num_kv_blocks
         if self.device.type != "cuda":
@@ -242,10 +269,9 @@ class LLMEngine:
         free, total = torch.cuda.mem_get_info(self.device)
         used = total - free
         budget = int(total * cfg.gpu_memory_utilization) - used - _RESERVE_BYTES
-        num = KVCache.num_blocks_for_budget(
-            budget, self.spec.num_layers, kv_heads_local, cfg.kv_block_size,
-            self.spec.head_dim, self.kv_dtype,
-        )
+        per_block = KVCache.layout_block_bytes(self.kv_layout, cfg.kv_block_size, self.kv_dtype)
+        num = max(budget // per_block, 0) if per_block else (
+            cfg.max_num_seqs * self.max_model_len) // cfg.kv_block_size + cfg.max_num_seqs
         # No point holding more KV than every admitted seq at full context.
         cap = (cfg.max_num_seqs * self.max_model_len) // cfg.kv_block_size + cfg.max_num_seqs
         num = min(num, cap)
@@ -296,15 +322,17 @@ class LLMEngine:
 
     last_step_kind: str = "decode"  # observability: kind of the last step
 
-    def step(self) -> List[RequestOutput]:
-        batch = self.scheduler.schedule()
-        if batch.empty:
-            return []
-        self.last_step_kind = batch.kind
-        t0 = time.perf_counter()
+    def _execute(self, batch, want=None) -> torch.Tensor:
+        """Run one scheduled batch: the sampled tokens of its sampling rows,
+        or (replay) the logits of the rows ``want`` names. ``want`` is
+        aligned with batch.seqs: per sequence, positions relative to the
+        tokens it runs this step."""
         if batch.kind == "prefill":
-            tokens = self.runner.execute_prefill(batch.seqs, batch.chunks or None)
-        elif batch.kind == "mixed":
+            return self.runner.execute_prefill(batch.seqs, batch.chunks or None, want=want)
+        if batch.kind == "mixed":
+            nd = batch.n_decode
+            wd = None if want is None else want[:nd]
+            wp = None if want is None else want[nd:]
             ptoks = sum(e - st for st, e in batch.chunks)
             if ptoks < _MIXED_FUSE_MIN_TOKENS and self.runner.use_graphs:
                 # SPLIT policy (default, measured fastest): replay the
@@ -315,8 +343,8 @@ class LLMEngine:
                 # concurrently (profiles/r2_step2). TP replicas stay
                 # sequential: stream interleaving would make rank-local
                 # RNG/collective ordering nondeterministic.
-                dseqs = batch.seqs[: batch.n_decode]
-                pseqs = batch.seqs[batch.n_decode :]
+                dseqs = batch.seqs[:nd]
+                pseqs = batch.seqs[nd:]
                 if self._overlap_mixed:
                     ds = self._decode_stream
                     cur = torch.cuda.current_stream()
@@ -324,24 +352,87 @@ class LLMEngine:
                     with torch.cuda.stream(ds):
                         # .clone(): the fused sampler returns a VIEW of a
                         # persistent output buffer
-                        d_tokens = self.runner.execute_decode(
-                            dseqs, force_eager=self._overlap_eager).clone()
+                        d_out = self.runner.execute_decode(
+                            dseqs, force_eager=self._overlap_eager, want=wd).clone()
                     if self._overlap_sync:
                         ds.synchronize()
-                    p_tokens = self.runner.execute_prefill(
-                        pseqs, batch.chunks, buf_name="prefill"
-                    )
+                    p_out = self.runner.execute_prefill(
+                        pseqs, batch.chunks, buf_name="prefill", want=wp)
                     cur.wait_stream(ds)
-                    d_tokens.record_stream(cur)
-                    tokens = torch.cat([d_tokens, p_tokens])
-                else:
-                    d_tokens = self.runner.execute_decode(dseqs).clone()
-                    p_tokens = self.runner.execute_prefill(pseqs, batch.chunks)
-                    tokens = torch.cat([d_tokens, p_tokens])
+                    d_out.record_stream(cur)
+                    return torch.cat([d_out, p_out])
+                d_out = self.runner.execute_decode(dseqs, want=wd).clone()
+                p_out = self.runner.execute_prefill(pseqs, batch.chunks, want=wp)
+                return torch.cat([d_out, p_out])
+            return self.runner.execute_mixed(batch, want=want)
+        return self.runner.execute_decode(batch.seqs, want=want)
+
+    # -- teacher-forced replay ---------------------------------------------
+
+    def replay_step(self, entries: List[dict], end: Optional[List[str]] = None) -> torch.Tensor:
+        """Feed given tokens instead of sampling. ``entries``: per request
+        {"id", "tokens", "want"} — its next tokens, and the positions among
+        them whose logits are wanted. All entries form ONE batch through the
+        scheduler's block/slot allocators and the runner's prefill / decode /
+        mixed paths (a request is admitted at its first entry and may skip
+        steps). Requests named in ``end`` release their blocks and state
+        slot after the step. Returns fp32 logits [wanted, vocab] in the
+        order of the entries and of their ``want``."""
+        plan, wants = [], {}
+        for ent in entries:
+            rid, toks = ent["id"], list(ent["tokens"])
+            if not toks:
+                raise ValueError(f"request {rid}: an entry needs at least one token")
+            seq = self._seqs.get(rid)
+            if seq is None:
+                if len(self._seqs) >= self.config.max_num_seqs:
+                    raise RuntimeError("more live requests than max_num_seqs")
+                seq = Sequence(rid, toks, SamplingParams(), arrival_time=time.time())
+                if len(toks) > self.max_model_len:
+                    raise ValueError(f"request {rid} exceeds max_model_len")
+                self._seqs[rid] = seq
             else:
-                tokens = self.runner.execute_mixed(batch)
-        else:
-            tokens = self.runner.execute_decode(batch.seqs)
+                seq.token_ids.extend(toks)
+                seq.prompt_len = len(seq.token_ids)
+            if seq.num_tokens > self.max_model_len:
+                raise ValueError(f"request {rid} exceeds max_model_len")
+            w = list(ent.get("want") or [])
+            if any(x < 0 or x >= len(toks) for x in w):
+                raise ValueError(f"request {rid}: wanted position outside the entry")
+            wants[rid] = w
+            plan.append((seq, len(toks)))
+        out = None
+        if plan:
+            batch = self.scheduler.schedule_plan(plan)
+            self.last_step_kind = batch.kind
+            logits = self._execute(batch, want=[wants[s.request_id] for s in batch.seqs])
+            self.steps += 1
+            for seq, n in plan:
+                seq.prefilled += n
+            # rows come back in batch order (decode rows first); return them
+            # in the order of the entries
+            offs, at = {}, 0
+            for s in batch.seqs:
+                offs[s.request_id] = (at, at + len(wants[s.request_id]))
+                at += len(wants[s.request_id])
+            order = [i for ent in entries for i in range(*offs[ent["id"]])]
+            out = logits[torch.tensor(order, dtype=torch.long, device=logits.device)] \
+                if order else logits[:0]
+        for rid in end or []:
+            seq = self._seqs.pop(rid, None)
+            if seq is not None:
+                self.scheduler.finish(seq, "replayed")
+        if out is None:
+            out = torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+        return out
+
+    def step(self) -> List[RequestOutput]:
+        batch = self.scheduler.schedule()
+        if batch.empty:
+            return []
+        self.last_step_kind = batch.kind
+        t0 = time.perf_counter()
+        tokens = self._execute(batch)
         token_list = tokens.tolist()
         now = time.time()
         self.steps += 1

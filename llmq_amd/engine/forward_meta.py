@@ -21,6 +21,17 @@ class ChunkGather:
 
 
 @dataclass
+class RecurrentMeta:
+    """Rows of a step grouped per sequence for recurrent layers: sequence b
+    owns rows [cu[b], cu[b+1]) and state slot slots[b]; fresh[b] != 0 means
+    its rows start at position 0 (the state starts from zero)."""
+
+    cu: torch.Tensor      # [B+1] int32
+    slots: torch.Tensor   # [B] int32
+    fresh: torch.Tensor   # [B] int32
+
+
+@dataclass
 class PrefillMeta:
     """Packed variable-length prompt batch (whole prompts or chunks)."""
 
@@ -28,6 +39,10 @@ class PrefillMeta:
     max_seqlen: int
     slot_mapping: torch.Tensor  # [T] int64 global KV slots
     gather: "ChunkGather | None" = None  # set when any entry is a chunk
+    # models whose prefill attention reads the paged cache directly:
+    block_tables: "torch.Tensor | None" = None  # [B, max_blocks] int32
+    q_start: "torch.Tensor | None" = None       # [B] int32 first query position
+    recurrent: "RecurrentMeta | None" = None
 
     is_prefill: bool = True
     is_mixed: bool = False
@@ -40,6 +55,7 @@ class DecodeMeta:
     block_tables: torch.Tensor  # [B, max_blocks] int32
     context_lens: torch.Tensor  # [B] int32 (including the new token)
     slot_mapping: torch.Tensor  # [B] int64
+    recurrent: "RecurrentMeta | None" = None
 
     is_prefill: bool = False
     is_mixed: bool = False
@@ -56,6 +72,7 @@ class MixedMeta:
     decode: "DecodeMeta"
     prefill: "PrefillMeta"
     slot_mapping: torch.Tensor  # [T] both segments, in row order
+    recurrent: "RecurrentMeta | None" = None  # over ALL rows, decode rows first
 
     is_prefill: bool = False
     is_mixed: bool = True

@@ -13,7 +13,7 @@ usual admission limit)."""
 from __future__ import annotations
 
 import logging
-from typing import List, Optional
+from typing import List, Optional, Tuple
 
 import torch
 
@@ -21,6 +21,11 @@ logger = logging.getLogger(__name__)
 
 
 class KVCache:
+    """Uniform models pass (num_layers, num_kv_heads, head_dim); models whose
+    layers differ pass ``layout``: one (kv_heads, k_dim, v_dim) per layer, or
+    None for a layer that caches no keys (its k/v entries are None). All
+    layers share block ids, so one block table serves every layer."""
+
     def __init__(
         self,
         num_layers: int,
@@ -30,28 +35,42 @@ class KVCache:
         head_dim: int,
         device: torch.device,
         dtype: torch.dtype,
+        layout: Optional[List[Optional[Tuple[int, int, int]]]] = None,
     ):
-        self.num_layers = num_layers
+        if layout is None:
+            layout = [(num_kv_heads, head_dim, head_dim)] * num_layers
+        self.layout = list(layout)
+        self.num_layers = len(self.layout)
         self.num_blocks = num_blocks
         self.block_size = block_size
-        self.k: List[torch.Tensor] = []
-        self.v: List[torch.Tensor] = []
-        for _ in range(num_layers):
+        # per-sequence recurrent state of the same model (set by the engine
+        # for models with recurrent layers): one cache object reaches forward
+        self.recurrent: Optional["RecurrentStateCache"] = None
+        self.k: List[Optional[torch.Tensor]] = []
+        self.v: List[Optional[torch.Tensor]] = []
+        for entry in self.layout:
+            if entry is None:
+                self.k.append(None)
+                self.v.append(None)
+                continue
+            heads, k_dim, v_dim = entry
             self.k.append(
-                torch.zeros(
-                    num_blocks, num_kv_heads, block_size, head_dim, device=device, dtype=dtype
-                )
+                torch.zeros(num_blocks, heads, block_size, k_dim, device=device, dtype=dtype)
             )
             self.v.append(
-                torch.zeros(
-                    num_blocks, num_kv_heads, block_size, head_dim, device=device, dtype=dtype
-                )
+                torch.zeros(num_blocks, heads, block_size, v_dim, device=device, dtype=dtype)
             )
 
     @staticmethod
     def block_bytes(num_layers, num_kv_heads, block_size, head_dim, dtype) -> int:
         elem = torch.tensor([], dtype=dtype).element_size()
         return 2 * num_layers * num_kv_heads * block_size * head_dim * elem
+
+    @staticmethod
+    def layout_block_bytes(layout, block_size, dtype) -> int:
+        elem = torch.tensor([], dtype=dtype).element_size()
+        return sum(h * block_size * (kd + vd) * elem for (h, kd, vd) in
+                   (e for e in layout if e is not None))
 
     @classmethod
     def num_blocks_for_budget(
@@ -90,3 +109,50 @@ class BlockAllocator:
 
 def blocks_needed(num_tokens: int, block_size: int) -> int:
     return (num_tokens + block_size - 1) // block_size
+
+
+class RecurrentStateCache:
+    """Per-sequence recurrent state, one fp32 tensor [num_slots + 1, *shape]
+    per recurrent layer (None for the others). A sequence owns one slot id
+    across all layers from admission to release; slot ``num_slots`` is a
+    scratch row for the padding rows of a captured decode graph. Slots are
+    never cleared: a sequence's first portion starts from zero by itself."""
+
+    def __init__(self, layout: List[Optional[Tuple[int, ...]]], num_slots: int,
+                 device: torch.device):
+        self.layout = list(layout)
+        self.num_slots = num_slots
+        self.pad_slot = num_slots
+        self.state: List[Optional[torch.Tensor]] = [
+            None if shape is None
+            else torch.zeros(num_slots + 1, *shape, device=device, dtype=torch.float32)
+            for shape in self.layout
+        ]
+
+    @property
+    def active(self) -> bool:
+        return any(s is not None for s in self.state)
+
+    def bytes(self) -> int:
+        return sum(s.numel() * 4 for s in self.state if s is not None)
+
+
+class SlotAllocator:
+    """Free-list over state slot ids [0, num_slots); lowest id first, so
+    released slots are handed out again at once."""
+
+    def __init__(self, num_slots: int):
+        self.num_slots = num_slots
+        self._free: List[int] = list(range(num_slots - 1, -1, -1))
+
+    @property
+    def num_free(self) -> int:
+        return len(self._free)
+
+    def allocate(self) -> Optional[int]:
+        return self._free.pop() if self._free else None
+
+    def free(self, slot: int) -> None:
+        if slot < 0 or slot >= self.num_slots or slot in self._free:
+            raise ValueError(f"bad state slot release: {slot}")
+        self._free.append(slot)

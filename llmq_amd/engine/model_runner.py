@@ -19,7 +19,9 @@ import torch
 
 from llmq_amd import ops
 from llmq_amd.engine.config import EngineConfig
-from llmq_amd.engine.forward_meta import ChunkGather, DecodeMeta, MixedMeta, PrefillMeta
+from llmq_amd.engine.forward_meta import (
+    ChunkGather, DecodeMeta, MixedMeta, PrefillMeta, RecurrentMeta,
+)
 from llmq_amd.engine.kv_cache import KVCache
 from llmq_amd.engine.models.llama import CausalLM
 from llmq_amd.engine.scheduler import ScheduledBatch, Sequence
@@ -64,6 +66,12 @@ class ModelRunner:
         # decode path, "prefill" for the prefill segment of an OVERLAPPED
         # split mixed step — two concurrent streams must not share them).
         self._sample_bufs: Dict[str, Dict[str, torch.Tensor]] = {}
+        # Models whose prompt-portion attention reads the paged cache through
+        # the block table (no gathered K/V copy), and models with recurrent
+        # layers (per-sequence state slots), get the extra step metadata.
+        self.paged_prefill = bool(getattr(model, "paged_prefill", False))
+        self.recurrent = kv_cache.recurrent if (
+            kv_cache.recurrent is not None and kv_cache.recurrent.active) else None
         if self.use_graphs:
             self._alloc_static_buffers()
 
@@ -80,6 +88,17 @@ class ModelRunner:
             B, self.max_blocks_per_seq, dtype=torch.int32, device=dev
         )
         self.in_context_lens = torch.ones(B, dtype=torch.int32, device=dev)
+        self.in_rec = None
+        if self.recurrent is not None:
+            # one row per sequence; slots are staged per step, rows never
+            # start a sequence (decode rows sit on cached context)
+            self.in_rec = RecurrentMeta(
+                cu=torch.arange(B + 1, dtype=torch.int32, device=dev),
+                slots=torch.full((B,), self.recurrent.pad_slot, dtype=torch.int32, device=dev),
+                fresh=torch.zeros(B, dtype=torch.int32, device=dev),
+            )
+            self.h_rec_slots = torch.zeros(B, dtype=torch.int32, pin_memory=True)
+            self.h_rec_fresh = torch.zeros(B, dtype=torch.int32, pin_memory=True)
         self.out_hidden = torch.zeros(
             B, self.model.spec.hidden_size, dtype=self.model.dtype, device=dev
         )
@@ -112,6 +131,16 @@ class ModelRunner:
                 context_lens=self.in_context_lens[:bs],
                 slot_mapping=self.in_slots[:bs],
             )
+            if self.in_rec is not None:
+                meta.recurrent = RecurrentMeta(
+                    cu=self.in_rec.cu[: bs + 1], slots=self.in_rec.slots[:bs],
+                    fresh=self.in_rec.fresh[:bs],
+                )
+                # capture and warmup rows write the scratch slot only
+                self.in_rec.slots.fill_(self.recurrent.pad_slot)
+                self.in_rec.fresh.fill_(1)
+            if self.paged_prefill:
+                self.in_slots.fill_(-1)  # capture/warmup rows enter no cache slot
             # warmup (also materialises workspace allocations)
             out = self.model.forward(self.in_ids[:bs], self.in_pos[:bs], self.kv_cache, meta)
             torch.cuda.synchronize()
@@ -150,7 +179,7 @@ class ModelRunner:
         cu = [0]
         cu_k = [0]
         rel_last: List[int] = []
-        any_chunk = any(start > 0 for (start, _e) in chunks)
+        any_chunk = (not self.paged_prefill) and any(start > 0 for (start, _e) in chunks)
         g_blocks: List[int] = []
         g_offs: List[int] = []
         past_dst: List[int] = []
@@ -192,12 +221,51 @@ class ModelRunner:
             slot_mapping=slot_mapping,
             gather=gather,
         )
+        if self.paged_prefill:
+            meta.block_tables = self._block_table_tensor(pseqs, dev)
+            meta.q_start = torch.tensor([st for (st, _e) in chunks], dtype=torch.int32, device=dev)
+        if self.recurrent is not None:
+            meta.recurrent = RecurrentMeta(
+                cu=meta.cu_seqlens,
+                slots=torch.tensor([s.state_slot for s in pseqs], dtype=torch.int32, device=dev),
+                fresh=torch.tensor([int(st == 0) for (st, _e) in chunks], dtype=torch.int32,
+                                   device=dev),
+            )
         return ids, pos, slot_mapping, meta, rel_last
 
+    def _block_table_tensor(self, seqs, dev) -> torch.Tensor:
+        width = max(1, max(len(s.block_table) for s in seqs))
+        bt_np = np.zeros((len(seqs), width), dtype=np.int32)
+        for i, s in enumerate(seqs):
+            bt_np[i, : len(s.block_table)] = s.block_table
+        return torch.from_numpy(bt_np).to(dev)
+
+    def _decode_recurrent_meta(self, seqs, dev):
+        if self.recurrent is None:
+            return None
+        n = len(seqs)
+        return RecurrentMeta(
+            cu=torch.arange(n + 1, dtype=torch.int32, device=dev),
+            slots=torch.tensor([s.state_slot for s in seqs], dtype=torch.int32, device=dev),
+            fresh=torch.zeros(n, dtype=torch.int32, device=dev),
+        )
+
+    def _logits_at(self, hidden: torch.Tensor, rows: List[int]) -> torch.Tensor:
+        """Logits of the given rows of a step (teacher-forced replay: the
+        caller asks for positions instead of sampling)."""
+        if not rows:
+            return torch.empty(0, self.model.spec.vocab_size, dtype=torch.float32,
+                               device=hidden.device)
+        idx = torch.tensor(rows, dtype=torch.long, device=hidden.device)
+        return self.model.compute_logits(hidden[idx]).float()
+
     @torch.no_grad()
-    def execute_prefill(self, seqs: List[Sequence], chunks=None, buf_name: str = "main") -> torch.Tensor:
+    def execute_prefill(self, seqs: List[Sequence], chunks=None, buf_name: str = "main",
+                        want=None) -> torch.Tensor:
         """Run a packed prefill segment; returns sampled next tokens for the
-        rows whose context completed this step (all rows when no chunking)."""
+        rows whose context completed this step (all rows when no chunking).
+        With ``want`` (per sequence, portion-relative positions) nothing is
+        sampled: the logits of those rows are returned, in that order."""
         if chunks is None:
             chunks = [(0, s.num_tokens) for s in seqs]
         dev = self.device
@@ -207,6 +275,11 @@ class ModelRunner:
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
         positions = torch.tensor(pos, dtype=torch.long, device=dev)
         hidden = self.model.forward(input_ids, positions, self.kv_cache, meta)
+        if want is not None:
+            cu = [0]
+            for st, e in chunks:
+                cu.append(cu[-1] + e - st)
+            return self._logits_at(hidden, [cu[b] + w for b, ws in enumerate(want) for w in ws])
         if not rel_last:
             return torch.empty(0, dtype=torch.long, device=dev)
         last_hidden = hidden[torch.tensor(rel_last, dtype=torch.long, device=dev)]
@@ -217,7 +290,7 @@ class ModelRunner:
     # -- mixed (decode rows + ride-along prefill rows, eager) ------------
 
     @torch.no_grad()
-    def execute_mixed(self, batch: "ScheduledBatch") -> torch.Tensor:
+    def execute_mixed(self, batch: "ScheduledBatch", want=None) -> torch.Tensor:
         """Decode seqs[:n_decode] and prefill seqs[n_decode:] in ONE forward:
         shared GEMMs/norms over the packed rows, per-segment attention.
         Runs eager (prefill shapes vary); pure-decode steps keep hipGraphs.
@@ -258,9 +331,24 @@ class ModelRunner:
             prefill=pmeta,
             slot_mapping=slot_mapping,
         )
+        if self.recurrent is not None:
+            dr, pr = self._decode_recurrent_meta(dseqs, dev), pmeta.recurrent
+            meta.decode.recurrent = dr
+            meta.recurrent = RecurrentMeta(
+                cu=torch.cat([dr.cu[:-1], pr.cu + nd]),
+                slots=torch.cat([dr.slots, pr.slots]),
+                fresh=torch.cat([dr.fresh, pr.fresh]),
+            )
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
         positions = torch.tensor(pos, dtype=torch.long, device=dev)
         hidden = self.model.forward(input_ids, positions, self.kv_cache, meta)
+        if want is not None:
+            cu = [nd]
+            for st, e in chunks:
+                cu.append(cu[-1] + e - st)
+            rows = [b for b, ws in enumerate(want[:nd]) if ws]
+            rows += [cu[b] + w for b, ws in enumerate(want[nd:]) for w in ws]
+            return self._logits_at(hidden, rows)
         last_idx = list(range(nd)) + [nd + r for r in rel_last]
         last_hidden = hidden[torch.tensor(last_idx, dtype=torch.long, device=dev)]
         logits = self.model.compute_logits(last_hidden)
@@ -272,7 +360,8 @@ class ModelRunner:
     # -- decode ----------------------------------------------------------
 
     @torch.no_grad()
-    def execute_decode(self, seqs: List[Sequence], force_eager: bool = False) -> torch.Tensor:
+    def execute_decode(self, seqs: List[Sequence], force_eager: bool = False,
+                       want=None) -> torch.Tensor:
         dev = self.device
         B = len(seqs)
         bs = self.block_size
@@ -283,7 +372,7 @@ class ModelRunner:
 
         bucket = self._bucket_for(B) if (self.use_graphs and not force_eager) else None
         if bucket is not None and bucket in self._graphs:
-            return self._decode_with_graph(seqs, bucket, ids, pos, slots, ctx)
+            return self._decode_with_graph(seqs, bucket, ids, pos, slots, ctx, want)
 
         block_tables = torch.zeros(
             B, max(len(s.block_table) for s in seqs), dtype=torch.int32, device=dev
@@ -296,15 +385,18 @@ class ModelRunner:
             block_tables=block_tables,
             context_lens=torch.tensor(ctx, dtype=torch.int32, device=dev),
             slot_mapping=torch.tensor(slots, dtype=torch.long, device=dev),
+            recurrent=self._decode_recurrent_meta(seqs, dev),
         )
         input_ids = torch.tensor(ids, dtype=torch.long, device=dev)
         positions = torch.tensor(pos, dtype=torch.long, device=dev)
         hidden = self.model.forward(input_ids, positions, self.kv_cache, meta)
+        if want is not None:
+            return self._logits_at(hidden, [b for b, ws in enumerate(want) if ws])
         logits = self.model.compute_logits(hidden)
         return self._sample(logits, seqs)
 
     def _decode_with_graph(
-        self, seqs: List[Sequence], bucket: int, ids, pos, slots, ctx
+        self, seqs: List[Sequence], bucket: int, ids, pos, slots, ctx, want=None
     ) -> torch.Tensor:
         B = len(seqs)
         # Stage metadata through pinned host buffers, one async copy each.
@@ -330,7 +422,8 @@ class ModelRunner:
         if B < bucket:
             # pad rows: context_len 1 pointing at block 0 (defined garbage,
             # their logits are never read)
-            self.h_slots[B:bucket] = 0
+            # padding rows of a paged-prefill model enter no cache slot at all
+            self.h_slots[B:bucket] = -1 if self.paged_prefill else 0
             self.h_ids[B:bucket] = 0
             self.h_pos[B:bucket] = 0
             for i in range(B, bucket):
@@ -344,7 +437,17 @@ class ModelRunner:
         self.in_block_tables[:bucket, :max_w].copy_(
             self.h_block_tables[:bucket, :max_w], non_blocking=True
         )
+        if self.in_rec is not None:
+            # padding rows advance the scratch slot from zero, never a live one
+            self.h_rec_slots[:B] = torch.tensor([s.state_slot for s in seqs], dtype=torch.int32)
+            self.h_rec_slots[B:bucket] = self.recurrent.pad_slot
+            self.h_rec_fresh[:B] = 0
+            self.h_rec_fresh[B:bucket] = 1
+            self.in_rec.slots[:bucket].copy_(self.h_rec_slots[:bucket], non_blocking=True)
+            self.in_rec.fresh[:bucket].copy_(self.h_rec_fresh[:bucket], non_blocking=True)
         self._graphs[bucket].replay()
+        if want is not None:
+            return self._logits_at(self.out_hidden[:B], [b for b, ws in enumerate(want) if ws])
         logits = self.model.compute_logits(self.out_hidden[:B])
         return self._sample(logits, seqs)
 

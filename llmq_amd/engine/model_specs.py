@@ -218,10 +218,176 @@ ALIASES = {
 }
 
 
+# ---------------------------------------------------------------------------
+# Hybrid decoders: a per-layer list of sequence mixers (block-local biased
+# attention, gated linear attention) with optional gated feed-forwards, an
+# fp32 residual stream and a zero-centred norm sandwich round every sublayer.
+
+
+@dataclass
+class BlockBiasAttnSpec:
+    """Attention whose keys are limited to the query's own span of `span`
+    positions (counted from position 0), with a learned bias per bucketed
+    distance, one RMSNorm over the whole q / k projection, optional value
+    blending with the first blending layer, and a sigmoid gate per head."""
+
+    heads: int
+    kv_heads: int
+    dim: int            # per-head q/k size
+    vdim: int           # per-head v size
+    scale: float
+    span: int           # mask span
+    bias_far: float     # distance at which the log buckets reach the last row
+    bias_rows: int = 16  # rows of the bias table (read from the tensor's shape)
+    v_mix: bool = False
+    kind: str = "attention"
+
+
+@dataclass
+class GLASpec:
+    """Gated linear attention: per head S ← diag(a) S + k vᵀ, o = Sᵀ q, with
+    a = sigmoid(low-rank(h) + b)^(1/tau) per key channel."""
+
+    heads: int
+    dim: int
+    vdim: int
+    tau: float
+    decay_rank: int = 16  # inner size of the decay projection (tensor shape)
+    kind: str = "gla"
+
+
+@dataclass
+class HybridLayerSpec:
+    mixer: object                 # BlockBiasAttnSpec | GLASpec
+    ff: int = 0                   # 0 = the layer has no feed-forward
+    ff_kind: str = "dense"
+
+
+@dataclass
+class HybridSpec:
+    name: str
+    family: str                   # "kakovik"
+    vocab_size: int
+    hidden_size: int
+    layers: list = field(default_factory=list)
+    rms_eps: float = 1e-6
+    logit_scale: float = 1.0
+    # no positional table: the limit only bounds block tables
+    max_position_embeddings: int = 1 << 17
+    tied_embeddings: bool = False
+    eos_token_id: int = 2
+    bos_token_id: int = 1
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def param_count(self) -> int:
+        w = self.hidden_size
+        total = 2 * self.vocab_size * w + w
+        for ls in self.layers:
+            m = ls.mixer
+            total += 2 * w
+            if m.kind == "attention":
+                nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
+                total += w * (nq + nk + nv + m.heads) + nq + nk
+                total += m.heads * m.vdim * w + m.bias_rows * m.heads + 1
+            else:
+                nk, nv = m.heads * m.dim, m.heads * m.vdim
+                total += w * (2 * nk + 2 * nv + m.decay_rank) + m.decay_rank * nk + nk
+                total += nv * w + m.vdim
+            if ls.ff:
+                total += 2 * w + 3 * w * ls.ff
+        return total
+
+
+def _safetensors_shapes(path: Path) -> dict:
+    """name → shape from a safetensors header (8-byte length + JSON); no
+    tensor data is read."""
+    import struct
+
+    with open(path, "rb") as fh:
+        (n,) = struct.unpack("<Q", fh.read(8))
+        header = json.loads(fh.read(n))
+    return {k: v["shape"] for k, v in header.items() if k != "__metadata__"}
+
+
+def kakovik_spec_from_config(cfg: dict, name: str, shapes: Optional[dict] = None) -> HybridSpec:
+    """Kakovik config.json → HybridSpec. Sizes the config does not carry
+    (bias-table rows, decay rank) come from the checkpoint's tensor shapes."""
+    shapes = shapes or {}
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc = lc["mixer"]
+        kind = lc["type"]
+        if kind == "attention":
+            rel = shapes.get(f"l{i}.mix.rel")
+            mixer = BlockBiasAttnSpec(
+                heads=mc["heads"], kv_heads=mc.get("kv_heads", mc["heads"]),
+                dim=mc["dim"], vdim=mc.get("vdim", mc["dim"]),
+                scale=float(mc["scale"]), span=int(mc["mask"]["size"]),
+                bias_far=float(mc["bias_max"]),
+                bias_rows=int(rel[0]) if rel else 16,
+                v_mix=bool(mc.get("v_mix", False)),
+            )
+        elif kind == "gla":
+            a1 = shapes.get(f"l{i}.mix.a1")
+            mixer = GLASpec(
+                heads=mc["heads"], dim=mc["dim"], vdim=mc.get("vdim", mc["dim"]),
+                tau=float(mc["tau"]), decay_rank=int(a1[0]) if a1 else 16,
+            )
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp = lc.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+        layers.append(HybridLayerSpec(mixer=mixer, ff=int(mlp["ff"]) if mlp else 0))
+    return HybridSpec(
+        name=name, family="kakovik", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers,
+        rms_eps=float(cfg["norm"]["eps"]), logit_scale=float(cfg.get("logit_scale", 1.0)),
+    )
+
+
+def _kakovik(name, vocab, width, n_layers, heads, kv_heads, dim, vdim, ff, span,
+             gla_every=3, gla_heads=None, gla_dim=None, gla_vdim=None, **kw):
+    """Preset builder: every `gla_every`-th layer is a gated-linear-attention
+    layer without feed-forward, the others attention + dense feed-forward."""
+    layers = []
+    for i in range(n_layers):
+        if gla_every and i % gla_every == gla_every - 1:
+            layers.append(HybridLayerSpec(GLASpec(
+                heads=gla_heads or heads, dim=gla_dim or dim, vdim=gla_vdim or vdim,
+                tau=16.0, decay_rank=16)))
+        else:
+            layers.append(HybridLayerSpec(BlockBiasAttnSpec(
+                heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5,
+                span=span, bias_far=float(span), bias_rows=32, v_mix=True), ff=ff))
+    return HybridSpec(name=name, family="kakovik", vocab_size=vocab, hidden_size=width,
+                      layers=layers, **kw)
+
+
+HYBRID_PRESETS = {
+    # CPU/GPU test config: unequal q/v sizes, grouped kv heads, short spans
+    "tiny-kakovik": _kakovik("tiny-kakovik", 512, 64, 3, 4, 2, 32, 16, 128, 24,
+                             gla_every=2, gla_heads=2, gla_dim=16, gla_vdim=32),
+    # benchmark configs at the layer sizes of llama-3.2-1b / -3b (the closest
+    # existing models): same width, heads, head size, feed-forward and depth
+    "kakovik-1b": _kakovik("kakovik-1b", 128256, 2048, 16, 32, 8, 64, 64, 8192, 2048,
+                           gla_every=4, gla_heads=16, gla_dim=64, gla_vdim=128),
+    "kakovik-3b": _kakovik("kakovik-3b", 128256, 3072, 28, 24, 8, 128, 128, 8192, 2048,
+                           gla_every=4, gla_heads=12, gla_dim=128, gla_vdim=256),
+}
+
+
 def spec_from_hf_config(path: Path, name: str) -> ModelSpec:
     """Build a spec from a HF checkpoint directory's config.json."""
     with open(path / "config.json", "r", encoding="utf-8") as fh:
         cfg = json.load(fh)
+    if str(cfg.get("architecture", "")).lower() == "kakovik":
+        st = path / "model.safetensors"
+        return kakovik_spec_from_config(
+            cfg, name, _safetensors_shapes(st) if st.is_file() else None)
     arch = (cfg.get("architectures") or [""])[0].lower()
     model_type = cfg.get("model_type", "").lower()
     if "gemma2" in arch or model_type == "gemma2":
@@ -293,7 +459,9 @@ def resolve_spec(model: str) -> ModelSpec:
     key = ALIASES.get(key, key)
     if key in PRESETS:
         return PRESETS[key]
+    if key in HYBRID_PRESETS:
+        return HYBRID_PRESETS[key]
     raise ValueError(
         f"Unknown model '{model}'. Provide a checkpoint directory with config.json "
-        f"or one of: {sorted(PRESETS) + sorted(ALIASES)}"
+        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(ALIASES)}"
     )

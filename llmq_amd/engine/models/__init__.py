@@ -1,3 +1,22 @@
+"""Model registry: spec family → model class."""
+
+from llmq_amd.engine.models.kakovik import KakovikLM
 from llmq_amd.engine.models.llama import CausalLM
 
-__all__ = ["CausalLM"]
+MODEL_CLASSES = {
+    "llama": CausalLM,
+    "qwen2": CausalLM,
+    "gemma2": CausalLM,
+    "mistral": CausalLM,
+    "kakovik": KakovikLM,
+}
+
+
+def model_class_for(spec):
+    try:
+        return MODEL_CLASSES[spec.family]
+    except KeyError:
+        raise ValueError(f"no model class registered for family {spec.family!r}") from None
+
+
+__all__ = ["CausalLM", "KakovikLM", "MODEL_CLASSES", "model_class_for"]

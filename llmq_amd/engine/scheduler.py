@@ -47,7 +47,7 @@ class Sequence:
         "request_id", "token_ids", "prompt_len", "params", "status",
         "block_table", "arrival_time", "first_token_time", "finish_reason",
         "output_text", "num_preemptions", "prefilled", "prefill_start_time",
-        "uid",
+        "uid", "state_slot",
     )
 
     def __init__(self, request_id: str, prompt_token_ids: List[int], params: SamplingParams,
@@ -70,6 +70,7 @@ class Sequence:
         self.num_preemptions = 0
         self.prefilled = 0  # context tokens whose KV is in the cache
         self.prefill_start_time: Optional[float] = None
+        self.state_slot = -1  # recurrent-state slot (models with recurrent layers)
 
     @property
     def num_tokens(self) -> int:
@@ -106,7 +107,11 @@ class Scheduler:
         max_num_seqs: int,
         max_prefill_tokens: int,
         max_model_len: int,
+        slot_allocator=None,
     ):
+        # models with recurrent layers: a sequence holds one state slot from
+        # admission to release (kv_cache.SlotAllocator); None = no such layers
+        self.slot_allocator = slot_allocator
         self.allocator = allocator
         self.block_size = block_size
         self.max_num_seqs = max_num_seqs
@@ -166,10 +171,11 @@ class Scheduler:
         seq.status = SeqStatus.FINISHED
         seq.finish_reason = reason
         self._release(seq)
-        try:
-            self.running.remove(seq)
-        except ValueError:
-            pass
+        for pool in (self.running, self.prefilling):
+            try:
+                pool.remove(seq)
+            except ValueError:
+                pass
 
     def schedule(self) -> ScheduledBatch:
         # One step = the decode batch (all running seqs) + a prefill segment
@@ -222,8 +228,11 @@ class Scheduler:
             end = min(n, budget)
             if end < n and prefills:
                 break  # start a long prompt's first chunk only at segment head
+            if not self._take_slot(seq):
+                break
             blocks = self.allocator.allocate(blocks_needed(end, bs))
             if blocks is None:
+                self._drop_slot(seq)
                 break
             seq.block_table = blocks
             seq.status = SeqStatus.RUNNING
@@ -251,6 +260,72 @@ class Scheduler:
         if seq.block_table:
             self.allocator.free(seq.block_table)
             seq.block_table = []
+        self._drop_slot(seq)
+
+    def _take_slot(self, seq: Sequence) -> bool:
+        if self.slot_allocator is None or seq.state_slot >= 0:
+            return True
+        slot = self.slot_allocator.allocate()
+        if slot is None:
+            return False
+        seq.state_slot = slot
+        return True
+
+    def _drop_slot(self, seq: Sequence) -> None:
+        if self.slot_allocator is not None and seq.state_slot >= 0:
+            self.slot_allocator.free(seq.state_slot)
+        seq.state_slot = -1
+
+    # -- replay: the caller dictates each step's portions ------------------
+
+    def schedule_plan(self, plan: List[tuple]) -> ScheduledBatch:
+        """Build one step from an explicit plan instead of the budget policy:
+        ``plan`` is [(seq, n_tokens)], each sequence running its next
+        n_tokens (already appended to seq.token_ids). A single token on top
+        of cached context is a decode row; anything else is a prefill
+        portion. Same allocators, block tables and batch layout as
+        schedule(); nothing is preempted — a plan the pool cannot hold
+        raises."""
+        decode: List[Sequence] = []
+        prefills: List[Sequence] = []
+        chunks: List[tuple] = []
+        bs = self.block_size
+        for seq, n in plan:
+            start, end = seq.prefilled, seq.prefilled + n
+            if n < 1 or end > seq.num_tokens:
+                raise ValueError(f"request {seq.request_id}: bad portion [{start}, {end})")
+            if seq.status == SeqStatus.WAITING:
+                try:
+                    self.waiting.remove(seq)
+                except ValueError:
+                    pass
+                if not self._take_slot(seq):
+                    raise RuntimeError("no free state slot for " + seq.request_id)
+                seq.status = SeqStatus.RUNNING
+            need = blocks_needed(end, bs) - len(seq.block_table)
+            if need > 0:
+                blocks = self.allocator.allocate(need)
+                if blocks is None:
+                    raise RuntimeError(
+                        f"KV pool exhausted: request {seq.request_id} needs {need} more "
+                        f"blocks, {self.allocator.num_free} free")
+                seq.block_table.extend(blocks)
+            if n == 1 and start > 0:
+                decode.append(seq)
+                if seq in self.prefilling:
+                    self.prefilling.remove(seq)
+                if seq not in self.running:
+                    self.running.append(seq)
+            else:
+                prefills.append(seq)
+                chunks.append((start, end))
+                if seq not in self.prefilling and seq not in self.running:
+                    self.prefilling.append(seq)
+        if not prefills:
+            return ScheduledBatch("decode", decode)
+        if not decode:
+            return ScheduledBatch("prefill", prefills, chunks=chunks)
+        return ScheduledBatch("mixed", decode + prefills, n_decode=len(decode), chunks=chunks)
 
 
     def _schedule_decode(self) -> ScheduledBatch:

@@ -32,6 +32,10 @@ def _shard_cols(t: torch.Tensor, rank: int, size: int) -> torch.Tensor:
 
 
 def load_safetensors_weights(model, path: Path) -> None:
+    loader = _FAMILY_LOADERS.get(model.spec.family)
+    if loader:
+        loader(model, path)
+        return
     from safetensors import safe_open  # noqa: PLC0415
 
     spec = model.spec
@@ -87,3 +91,72 @@ def load_safetensors_weights(model, path: Path) -> None:
         else:
             copy_(lw.pre_mlp_norm, get(p + "post_attention_layernorm.weight"))
     logger.info("loaded %d tensors from %s", len(tensors), path)
+
+
+def load_kakovik_weights(model, path: Path) -> None:
+    """Kakovik checkpoint names → the packed in-tree tensors.
+
+    Checkpoint: 'embed', 'head', 'final.norm', and per layer 'l<i>.norm1',
+    'l<i>.norm1b' (+ 'norm2', 'norm2b' with a feed-forward), the mixer under
+    'l<i>.mix.' and the feed-forward under 'l<i>.mlp.'; linear weights are
+    [out, in]. Packing: attention q‖k‖v‖g → qkvg, GLA q‖k‖v‖g‖a1 → qkvga,
+    feed-forward gate‖up → gate_up."""
+    from safetensors import safe_open  # noqa: PLC0415
+
+    files = sorted(path.glob("*.safetensors"))
+    if not files:
+        raise FileNotFoundError(f"no .safetensors under {path}")
+    tensors: Dict[str, torch.Tensor] = {}
+    for f in files:
+        with safe_open(str(f), framework="pt", device="cpu") as sf:
+            for name in sf.keys():
+                tensors[name] = sf.get_tensor(name)
+    used = set()
+
+    def get(name: str) -> torch.Tensor:
+        if name not in tensors:
+            raise KeyError(f"missing tensor {name}")
+        used.add(name)
+        return tensors[name]
+
+    def copy_(dst: torch.Tensor, src: torch.Tensor) -> None:
+        if dst.shape != src.shape:
+            raise ValueError(f"shape mismatch: {tuple(dst.shape)} vs {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    copy_(model.embedding, get("embed"))
+    copy_(model.lm_head, get("head"))
+    copy_(model.final_norm, get("final.norm"))
+    for i, (ls, lw) in enumerate(zip(model.spec.layers, model.layers)):
+        p, t = f"l{i}.", lw.t
+        copy_(t["norm1"], get(p + "norm1"))
+        copy_(t["norm1b"], get(p + "norm1b"))
+        mx = p + "mix."
+        if ls.mixer.kind == "attention":
+            copy_(t["qkvg"], torch.cat([get(mx + "q"), get(mx + "k"), get(mx + "v"),
+                                        get(mx + "g")], dim=0))
+            copy_(t["q_norm"], get(mx + "q.norm"))
+            copy_(t["k_norm"], get(mx + "k.norm"))
+            copy_(t["rel"], get(mx + "rel"))
+            copy_(t["vmix"], get(mx + "vmix"))
+            copy_(t["o"], get(mx + "o"))
+        else:
+            copy_(t["qkvga"], torch.cat([get(mx + "q"), get(mx + "k"), get(mx + "v"),
+                                         get(mx + "g"), get(mx + "a1")], dim=0))
+            copy_(t["a2"], get(mx + "a2"))
+            copy_(t["a2_b"], get(mx + "a2.b"))
+            copy_(t["norm"], get(mx + "norm"))
+            copy_(t["o"], get(mx + "o"))
+        if ls.ff:
+            copy_(t["norm2"], get(p + "norm2"))
+            copy_(t["norm2b"], get(p + "norm2b"))
+            copy_(t["gate_up"], torch.cat([get(p + "mlp.gate"), get(p + "mlp.up")], dim=0))
+            copy_(t["down"], get(p + "mlp.down"))
+    unused = sorted(set(tensors) - used)
+    if unused:
+        raise ValueError(f"checkpoint tensors the model does not know: {unused[:8]}")
+    model.finalize()
+    logger.info("loaded %d tensors from %s", len(tensors), path)
+
+
+_FAMILY_LOADERS = {"kakovik": load_kakovik_weights}

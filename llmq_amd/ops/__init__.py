@@ -331,3 +331,142 @@ def _sample_tokens_gpu(
     sampled = (scaled + gumbel).argmax(dim=-1)
     greedy_choice = logits.argmax(dim=-1)
     return torch.where(greedy, greedy_choice, sampled)
+
+
+# ------------------------------------------------------ hybrid decoders --
+# Ops of the hybrid-decoder families (fp32 residual stream, block-local
+# biased attention, gated-linear-attention recurrences). They live in a
+# library of their own (_hip_hybrid*.so), loaded on first use; the same
+# policy applies: on a GPU the HIP kernels run or the op raises.
+
+_HY = None
+_HY_ERROR: Optional[str] = None
+_HY_TRIED = False
+
+
+def _try_load_hybrid() -> None:
+    global _HY, _HY_ERROR, _HY_TRIED
+    if _HY_TRIED:
+        return
+    _HY_TRIED = True
+    here = Path(__file__).parent
+    override = os.environ.get("LLMQ_HYBRID_OPS_SO")
+    candidates = [Path(override)] if override else sorted(here.glob("_hip_hybrid*.so"))
+    if not candidates:
+        _HY_ERROR = (
+            f"hybrid HIP extension not built (no _hip_hybrid*.so under {here}). "
+            "Run `python -m llmq_amd.ops.build --group hybrid`."
+        )
+        return
+    try:
+        torch.ops.load_library(str(candidates[0]))
+        _HY = torch.ops.llmq_amd_hybrid
+    except Exception as exc:  # noqa: BLE001
+        try:
+            torch.ops.llmq_amd_hybrid.rmsnorm_cast  # noqa: B018
+            _HY = torch.ops.llmq_amd_hybrid
+        except Exception:
+            _HY_ERROR = f"failed to load {candidates[0]}: {exc}"
+
+
+def has_hybrid_ext() -> bool:
+    _try_load_hybrid()
+    return _HY is not None
+
+
+def _use_hybrid(t: torch.Tensor) -> bool:
+    if not t.is_cuda:
+        return False
+    _try_load_hybrid()
+    if _HY is None:
+        raise RuntimeError(
+            f"llmq_amd hybrid HIP extension required for GPU execution but unavailable: {_HY_ERROR}"
+        )
+    return True
+
+
+def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    """RMSNorm of x (fp32 stream or model dtype) written in out_dtype."""
+    if _use_hybrid(x):
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+        _HY.rmsnorm_cast(out, x, weight, eps, offset)
+        return out
+    return torch_ref.rmsnorm_cast(x, weight, eps, offset, out_dtype)
+
+
+def sandwich_norm_res32(x: torch.Tensor, residual: torch.Tensor, w_post: torch.Tensor,
+                        w_pre: torch.Tensor, eps: float, offset: float) -> torch.Tensor:
+    """residual (fp32, in place) += rmsnorm(x)·(w_post+offset); returns
+    rmsnorm(residual)·(w_pre+offset) in x's dtype (x's storage on GPU)."""
+    if _use_hybrid(x):
+        _HY.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset)
+        return x
+    return torch_ref.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset)
+
+
+def act_and_mul(x: torch.Tensor, gelu: bool = False) -> torch.Tensor:
+    """[*, 2d] → act(x[..., :d]) · x[..., d:], act = SiLU or tanh-GELU."""
+    if _use_hybrid(x):
+        d = x.shape[-1] // 2
+        out = torch.empty(*x.shape[:-1], d, dtype=x.dtype, device=x.device)
+        _HY.act_and_mul(out, x, gelu)
+        return out
+    return torch_ref.act_and_mul(x, gelu)
+
+
+def qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, lam: float, k_cache, v_cache,
+                      slot_mapping, eps: float) -> None:
+    """Whole-projection RMSNorm of q (in place) and k, value blending with an
+    earlier layer's values, and the paged-cache scatter of k and v — fused."""
+    if _use_hybrid(q):
+        _HY.qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, float(lam), k_cache, v_cache,
+                              slot_mapping, eps)
+        return
+    torch_ref.qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, lam, k_cache, v_cache,
+                                slot_mapping, eps)
+
+
+def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q, q_start,
+                            max_q: int, span: int, scale: float) -> torch.Tensor:
+    """Block-local causal attention + per-distance bias for packed prompt
+    portions; keys/values come from the paged cache. q [T, H, D] → [T, H, DV]."""
+    if _use_hybrid(q):
+        out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
+        _HY.chunk_bias_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
+                                    q_start, int(max_q), int(span), float(scale))
+        return out
+    return torch_ref.chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables,
+                                             cu_q, q_start, span, scale)
+
+
+def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, context_lens,
+                           span: int, scale: float) -> torch.Tensor:
+    """The single-token form: query b sits at position context_lens[b]-1."""
+    if _use_hybrid(q):
+        out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
+        _HY.chunk_bias_attn_decode(out, q, gate, k_cache, v_cache, bias, block_tables,
+                                   context_lens, int(span), float(scale))
+        return out
+    return torch_ref.chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables,
+                                            context_lens, span, scale)
+
+
+def gla_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau: float) -> torch.Tensor:
+    """Gated-linear-attention recurrence over packed sequences; returns o
+    [T, H, DV] fp32 and advances state [slots, H, D, DV] in place."""
+    if _use_hybrid(q):
+        o = torch.empty(q.shape[0], q.shape[1], v.shape[2], dtype=torch.float32, device=q.device)
+        _HY.gla_recurrence(o, q, k, v, z, z_bias, state, cu, slots, fresh, float(tau))
+        return o
+    return torch_ref.gla_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau)
+
+
+def gla_out_norm_gate(o, weight, gate, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-head RMSNorm of the recurrence output × weight × SiLU(gate)."""
+    if _use_hybrid(o):
+        T, H, DV = o.shape
+        out = torch.empty(T, H * DV, dtype=out_dtype, device=o.device)
+        _HY.gla_out_norm_gate(out, o, weight, gate, eps)
+        return out
+    return torch_ref.gla_out_norm_gate(o, weight, gate, eps, out_dtype)

@@ -1,0 +1,500 @@
+// Sequence-mixer kernels for hybrid decoders (gfx950): layers that keep the
+// residual stream in fp32, block-local ("chunked") attention with a learned
+// per-distance bias over the paged KV cache, and gated-linear-attention
+// recurrences over per-sequence fp32 state slots.
+//
+// Numerics contract shared by every kernel here: activations arrive in the
+// model dtype T (bf16 or fp32); norms, scores, softmax weights, decays and
+// recurrent state are fp32 in registers/LDS and rounded to T once, on store.
+
+#include "common.h"
+
+// ------------------------------------------------------------------ norms --
+// Residual stream in fp32, sublayer I/O in T.
+
+// out = rmsnorm(in) * (w + offset); TI/TO may differ (fp32 stream -> T).
+template <typename TI, typename TO>
+__global__ void rmsnorm_cast_kernel(TO* __restrict__ out, const TI* __restrict__ in,
+                                    const TO* __restrict__ weight, int hidden,
+                                    float eps, float offset) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  const TI* x = in + row * hidden;
+  TO* o = out + row * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float f = to_f32(x[i]);
+    ss += f * f;
+  }
+  ss = block_reduce_sum(ss, red);
+  const float inv = 1.0f / sqrtf(ss / hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    o[i] = from_f32<TO>(to_f32(x[i]) * inv * (to_f32(weight[i]) + offset));
+}
+
+// Norm sandwich around an fp32 residual:
+//   residual += rmsnorm(x) * (w_post + offset)        (fp32, in place)
+//   x         = rmsnorm(residual) * (w_pre + offset)  (T, in place)
+// One launch closes a sublayer and opens the next.
+template <typename T>
+__global__ void sandwich_norm_res32_kernel(T* __restrict__ x, float* __restrict__ residual,
+                                           const T* __restrict__ w_post,
+                                           const T* __restrict__ w_pre, int hidden,
+                                           float eps, float offset) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  T* xr = x + row * hidden;
+  float* rr = residual + row * hidden;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float f = to_f32(xr[i]);
+    ss += f * f;
+  }
+  ss = block_reduce_sum(ss, red);
+  const float inv1 = 1.0f / sqrtf(ss / hidden + eps);
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float r = rr[i] + to_f32(xr[i]) * inv1 * (to_f32(w_post[i]) + offset);
+    rr[i] = r;
+    ss2 += r * r;
+  }
+  ss2 = block_reduce_sum(ss2, red);
+  const float inv2 = 1.0f / sqrtf(ss2 / hidden + eps);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x)
+    xr[i] = from_f32<T>(rr[i] * inv2 * (to_f32(w_pre[i]) + offset));
+}
+
+// ------------------------------------------------------------ activations --
+// Scalar fallback of act_and_mul for widths that are not a multiple of the
+// 16-byte vector (the vector kernel lives in elementwise.hip).
+template <typename T, bool GELU>
+__global__ void act_and_mul_scalar_kernel(T* __restrict__ out, const T* __restrict__ in,
+                                          long rows, int d) {
+  const long total = rows * d;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long row = idx / d;
+    const int col = (int)(idx % d);
+    const float g = to_f32(in[row * 2 * d + col]);
+    const float u = to_f32(in[row * 2 * d + d + col]);
+    float act;
+    if (GELU) {
+      const float c = 0.7978845608028654f;
+      act = 0.5f * g * (1.0f + tanhf(c * (g + 0.044715f * g * g * g)));
+    } else {
+      act = g / (1.0f + expf(-g));
+    }
+    out[idx] = from_f32<T>(act * u);
+  }
+}
+
+// ------------------------------------------------- attention: projections --
+// Per token: RMS-normalise the WHOLE q projection and the WHOLE k projection
+// (all heads at once, plain weights), blend v with an earlier layer's values
+// of the same token, and scatter k / v into the paged cache. q is normalised
+// in place; k and v are only read (attention reads them back from the cache).
+// Cache layouts: k [blocks, G, bs, D], v [blocks, G, bs, DV].
+template <typename T>
+__global__ void qknorm_vmix_cache_kernel(
+    T* __restrict__ q, long q_stride, int nq,
+    const T* __restrict__ k, long k_stride, int nk,
+    const T* __restrict__ v, long v_stride, int nv,
+    const T* __restrict__ q_w, const T* __restrict__ k_w,
+    const T* __restrict__ v_first, long vf_stride, float lambda,
+    T* __restrict__ k_cache, T* __restrict__ v_cache,
+    const long* __restrict__ slots, int kv_heads, int dim, int vdim,
+    int block_size, float eps) {
+  __shared__ float red[4];
+  const long tok = blockIdx.x;
+  T* qr = q + tok * q_stride;
+  const T* kr = k + tok * k_stride;
+  const T* vr = v + tok * v_stride;
+  float sq = 0.f, sk = 0.f;
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    const float f = to_f32(qr[i]);
+    sq += f * f;
+  }
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const float f = to_f32(kr[i]);
+    sk += f * f;
+  }
+  sq = block_reduce_sum(sq, red);
+  sk = block_reduce_sum(sk, red);
+  const float iq = 1.0f / sqrtf(sq / nq + eps);
+  const float ik = 1.0f / sqrtf(sk / nk + eps);
+  for (int i = threadIdx.x; i < nq; i += blockDim.x)
+    qr[i] = from_f32<T>(to_f32(qr[i]) * iq * to_f32(q_w[i]));
+  const long slot = slots[tok];
+  if (slot < 0) return;  // padding row: nothing enters the cache
+  const long blk = slot / block_size;
+  const int off = (int)(slot % block_size);
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const int g = i / dim, d = i % dim;
+    k_cache[((blk * kv_heads + g) * block_size + off) * dim + d] =
+        from_f32<T>(to_f32(kr[i]) * ik * to_f32(k_w[i]));
+  }
+  const T* vf = v_first ? v_first + tok * vf_stride : nullptr;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    const int g = i / vdim, d = i % vdim;
+    float val = to_f32(vr[i]);
+    if (vf) val = (1.0f - lambda) * val + lambda * to_f32(vf[i]);
+    v_cache[((blk * kv_heads + g) * block_size + off) * vdim + d] = from_f32<T>(val);
+  }
+}
+
+// ---------------------------------------------- attention: prompt portions --
+// Block-local causal attention with a per-distance bias, queries packed
+// [Tq, H, D], keys/values read from the paged cache through the block table
+// (the portion's own rows were scattered there first), so a prompt cut at
+// any position sees exactly the keys a whole prompt would.
+//
+// Query i (absolute position) sees key j iff j <= i and j / block == i / block
+// ("block" = the mask's span, counted from position 0). score = q.k * scale +
+// bias[i - j, h]; softmax over the visible keys; the head's output is
+// multiplied by sigmoid(gate[i, h]).
+//
+// Workgroup = 16 query rows x 1 head, 4 waves x 4 rows. Key tiles of 64 are
+// staged in LDS as fp32; in the score phase a lane owns one key (4 rows
+// register-blocked), in the PV phase a lane owns value channels.
+constexpr int kAttnQT = 16;
+constexpr int kAttnKT = 64;
+
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
+    T* __restrict__ out, long out_stride,
+    const T* __restrict__ q, long q_stride,
+    const T* __restrict__ gate, long g_stride,
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const float* __restrict__ bias,        // [span, H]
+    const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_q,          // [B+1]
+    const int* __restrict__ q_start,       // [B] position of a sequence's first query
+    int H, int G, int D, int DV, int block_size, int span, float scale) {
+  extern __shared__ float smem[];
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int row0 = cu_q[b];
+  const int nq = cu_q[b + 1] - row0;
+  const int r0 = blockIdx.x * kAttnQT;
+  if (r0 >= nq) return;
+  const int rows = min(kAttnQT, nq - r0);
+  const int pos0 = q_start[b] + r0;
+  const int pos_last = pos0 + rows - 1;
+  const int g = h / (H / G);
+  const int DP = D + 1;
+  float* Ks = smem;                         // [KT][D+1]
+  float* Vs = Ks + kAttnKT * DP;            // [KT][DV]
+  float* Qs = Vs + kAttnKT * DV;            // [QT][D]
+  float* Ps = Qs + kAttnQT * D;             // [QT][KT]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+
+  for (int idx = tid; idx < kAttnQT * D; idx += 256) {
+    const int r = idx / D, d = idx % D;
+    Qs[idx] = r < rows
+        ? to_f32(q[(long)(row0 + r0 + r) * q_stride + (long)h * D + d]) * scale
+        : 0.f;
+  }
+  float m[4], l[4], acc[4][NV];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m[r] = -INFINITY;
+    l[r] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) acc[r][n] = 0.f;
+  }
+  const int* bt = block_tables + (long)b * bt_stride;
+  const int lo = (pos0 / span) * span;
+  for (int kt = lo; kt <= pos_last; kt += kAttnKT) {
+    const int nk = min(kAttnKT, pos_last + 1 - kt);
+    __syncthreads();
+    for (int idx = tid; idx < nk * D; idx += 256) {
+      const int jj = idx / D, d = idx % D;
+      const int key = kt + jj;
+      const long base = (((long)bt[key / block_size] * G + g) * block_size +
+                         key % block_size);
+      Ks[jj * DP + d] = to_f32(k_cache[base * D + d]);
+    }
+    for (int idx = tid; idx < nk * DV; idx += 256) {
+      const int jj = idx / DV, d = idx % DV;
+      const int key = kt + jj;
+      const long base = (((long)bt[key / block_size] * G + g) * block_size +
+                         key % block_size);
+      Vs[jj * DV + d] = to_f32(v_cache[base * DV + d]);
+    }
+    __syncthreads();
+    // scores: lane = key, 4 rows at once
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    const int key = kt + lane;
+    if (lane < nk) {
+      const float* kr = Ks + lane * DP;
+      const float* q0 = Qs + (w * 4) * D;
+      for (int d = 0; d < D; ++d) {
+        const float kd = kr[d];
+        s[0] += q0[d] * kd;
+        s[1] += q0[D + d] * kd;
+        s[2] += q0[2 * D + d] * kd;
+        s[3] += q0[3 * D + d] * kd;
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int i = pos0 + w * 4 + r;
+      const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
+                       key / span == i / span;
+      const float sc = vis ? s[r] + bias[(long)(i - key) * H + h] : -INFINITY;
+      const float tmax = wave_reduce_max(sc);
+      const float m_new = fmaxf(m[r], tmax);
+      float p = 0.f, corr = 1.f;
+      if (m_new > -INFINITY) {
+        corr = expf(m[r] - m_new);  // m[r] = -inf -> 0
+        p = vis ? expf(sc - m_new) : 0.f;
+      }
+      l[r] = l[r] * corr + wave_reduce_sum(p);
+#pragma unroll
+      for (int n = 0; n < NV; ++n) acc[r][n] *= corr;
+      m[r] = m_new;
+      Ps[(w * 4 + r) * kAttnKT + lane] = p;
+    }
+    __syncthreads();
+    // PV: lane = value channel
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int c = lane + 64 * n;
+      if (c < DV) {
+        const float* p0 = Ps + (w * 4) * kAttnKT;
+        float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
+        for (int jj = 0; jj < nk; ++jj) {
+          const float vv = Vs[jj * DV + c];
+          a0 += p0[jj] * vv;
+          a1 += p0[kAttnKT + jj] * vv;
+          a2 += p0[2 * kAttnKT + jj] * vv;
+          a3 += p0[3 * kAttnKT + jj] * vv;
+        }
+        acc[0][n] += a0;
+        acc[1][n] += a1;
+        acc[2][n] += a2;
+        acc[3][n] += a3;
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int rr = w * 4 + r;
+    if (rr >= rows) continue;
+    const long trow = row0 + r0 + rr;
+    float gs = 1.f;
+    if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[trow * g_stride + h])));
+    const float inv = gs / l[r];
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int c = lane + 64 * n;
+      if (c < DV) out[trow * out_stride + (long)h * DV + c] = from_f32<T>(acc[r][n] * inv);
+    }
+  }
+}
+
+// ------------------------------------------------ attention: single tokens --
+// One workgroup per (sequence, head); the query is the sequence's newest
+// token (position ctx-1). Waves take key tiles of 64 round-robin, each with
+// its own online softmax; partials merge through LDS.
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
+    T* __restrict__ out, long out_stride,
+    const T* __restrict__ q, long q_stride,
+    const T* __restrict__ gate, long g_stride,
+    const T* __restrict__ k_cache, const T* __restrict__ v_cache,
+    const float* __restrict__ bias,
+    const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ context_lens,
+    int H, int G, int D, int DV, int block_size, int span, float scale) {
+  extern __shared__ float smem[];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int g = h / (H / G);
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  float* Qs = smem;                    // [D]
+  float* Ps = Qs + D;                  // [4][64]
+  float* Ms = Ps + 4 * 64;             // [4] max, [4] sum
+  float* As = Ms + 8;                  // [4][DV]
+  for (int d = tid; d < D; d += 256)
+    Qs[d] = to_f32(q[(long)b * q_stride + (long)h * D + d]) * scale;
+  __syncthreads();
+  const int i = context_lens[b] - 1;
+  const int lo = (i / span) * span;
+  const int* bt = block_tables + (long)b * bt_stride;
+  float m = -INFINITY, l = 0.f, acc[NV];
+#pragma unroll
+  for (int n = 0; n < NV; ++n) acc[n] = 0.f;
+  for (int kt = lo + w * 64; kt <= i; kt += 4 * 64) {
+    const int nk = min(64, i + 1 - kt);
+    const int key = kt + lane;
+    long base = 0;
+    float sc = -INFINITY;
+    if (lane < nk) {
+      base = ((long)bt[key / block_size] * G + g) * block_size + key % block_size;
+      const T* kr = k_cache + base * D;
+      float s = 0.f;
+      for (int d = 0; d < D; ++d) s += Qs[d] * to_f32(kr[d]);
+      sc = s + bias[(long)(i - key) * H + h];
+    }
+    const float m_new = fmaxf(m, wave_reduce_max(sc));  // nk >= 1: finite
+    const float corr = expf(m - m_new);
+    const float p = lane < nk ? expf(sc - m_new) : 0.f;
+    l = l * corr + wave_reduce_sum(p);
+    m = m_new;
+    for (int jj = 0; jj < nk; ++jj) {
+      const float pj = __shfl(p, jj, WAVE);
+      const long vb = __shfl(base, jj, WAVE);
+      const T* vr = v_cache + vb * DV;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) {
+        const int c = lane + 64 * n;
+        if (jj == 0) acc[n] *= corr;
+        if (c < DV) acc[n] += pj * to_f32(vr[c]);
+      }
+    }
+  }
+  if (lane == 0) {
+    Ms[w] = m;
+    Ms[4 + w] = l;
+  }
+#pragma unroll
+  for (int n = 0; n < NV; ++n) {
+    const int c = lane + 64 * n;
+    if (c < DV) As[w * DV + c] = acc[n];
+  }
+  __syncthreads();
+  float mm = fmaxf(fmaxf(Ms[0], Ms[1]), fmaxf(Ms[2], Ms[3]));
+  float f[4], ll = 0.f;
+#pragma unroll
+  for (int ww = 0; ww < 4; ++ww) {
+    f[ww] = Ms[ww] > -INFINITY ? expf(Ms[ww] - mm) : 0.f;
+    ll += Ms[4 + ww] * f[ww];
+  }
+  float gs = 1.f;
+  if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[(long)b * g_stride + h])));
+  for (int c = tid; c < DV; c += 256) {
+    const float a = As[c] * f[0] + As[DV + c] * f[1] + As[2 * DV + c] * f[2] +
+                    As[3 * DV + c] * f[3];
+    out[(long)b * out_stride + (long)h * DV + c] = from_f32<T>(a * gs / ll);
+  }
+}
+
+// ----------------------------------------------- gated linear attention ----
+// Per head, per sequence: S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t
+// with a_t = sigmoid(z_t + z_bias)^(1/tau) per key channel, state S in fp32
+// [D, DV] living in a per-sequence slot between steps.
+//
+// Value columns evolve independently, so the grid splits DV: a wave owns 16
+// columns, its lanes are 16 columns x 4 key groups (key channel d = kg + 4 i
+// sits in register S[i]); o is a 4-lane shuffle reduce. The workgroup's 4
+// waves share 16-token stages of q, k, decay (computed once, fp32) and v in
+// LDS. Sequential over tokens, parallel over (sequence, head, 64 columns).
+// A sequence whose portion starts at position 0 (fresh != 0) starts from a
+// zero state without reading its slot, so reused slots need no clearing.
+constexpr int kGlaTB = 16;
+
+template <typename T, int DPL>
+__global__ __launch_bounds__(256) void gla_recurrence_kernel(
+    float* __restrict__ o,                  // [T, H, DV] fp32
+    const T* __restrict__ q, long q_stride,
+    const T* __restrict__ k, long k_stride,
+    const T* __restrict__ v, long v_stride,
+    const T* __restrict__ z, long z_stride,
+    const float* __restrict__ z_bias,       // [H*D]
+    float* __restrict__ state,              // [slots, H, D, DV]
+    const int* __restrict__ cu,             // [B+1] row offsets
+    const int* __restrict__ slots,          // [B]
+    const int* __restrict__ fresh,          // [B]
+    int H, int D, int DV, float inv_tau, float q_scale) {
+  extern __shared__ float smem[];
+  float* qs = smem;                 // [TB][D]
+  float* ks = qs + kGlaTB * D;      // [TB][D]
+  float* as = ks + kGlaTB * D;      // [TB][D]
+  float* vs = as + kGlaTB * D;      // [TB][64]
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int col = (lane & 15) + 16 * w;      // column within the 64-wide tile
+  const int c = blockIdx.x * 64 + col;
+  const int kg = lane >> 4;
+  const int row0 = cu[b];
+  const int n = cu[b + 1] - row0;
+  const long sbase = ((long)slots[b] * H + h) * D * (long)DV;
+  float S[DPL];
+  const bool use_old = fresh[b] == 0;
+#pragma unroll
+  for (int i = 0; i < DPL; ++i) {
+    const int d = kg + 4 * i;
+    S[i] = (use_old && d < D && c < DV) ? state[sbase + (long)d * DV + c] : 0.f;
+  }
+  for (int t0 = 0; t0 < n; t0 += kGlaTB) {
+    const int nt = min(kGlaTB, n - t0);
+    __syncthreads();
+    for (int idx = tid; idx < nt * D; idx += 256) {
+      const int tt = idx / D, d = idx % D;
+      const long row = row0 + t0 + tt;
+      qs[idx] = to_f32(q[row * q_stride + (long)h * D + d]) * q_scale;
+      ks[idx] = to_f32(k[row * k_stride + (long)h * D + d]);
+      const float zz = to_f32(z[row * z_stride + (long)h * D + d]) + z_bias[h * D + d];
+      // log sigmoid(zz) = -(max(-zz, 0) + log1p(exp(-|zz|)))
+      const float ls = -(fmaxf(-zz, 0.f) + log1pf(expf(-fabsf(zz))));
+      as[idx] = expf(ls * inv_tau);
+    }
+    for (int idx = tid; idx < nt * 64; idx += 256) {
+      const int tt = idx >> 6, cc = idx & 63;
+      const int gc = blockIdx.x * 64 + cc;
+      vs[idx] = gc < DV
+          ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc])
+          : 0.f;
+    }
+    __syncthreads();
+    for (int tt = 0; tt < nt; ++tt) {
+      const float vv = vs[tt * 64 + col];
+      const float* qa = qs + tt * D;
+      const float* ka = ks + tt * D;
+      const float* aa = as + tt * D;
+      float part = 0.f;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int d = kg + 4 * i;
+        if (d < D) {
+          S[i] = aa[d] * S[i] + ka[d] * vv;
+          part += S[i] * qa[d];
+        }
+      }
+      part += __shfl_xor(part, 16, WAVE);
+      part += __shfl_xor(part, 32, WAVE);
+      if (kg == 0 && c < DV)
+        o[((long)(row0 + t0 + tt) * H + h) * DV + c] = part;
+    }
+  }
+  if (c < DV) {
+#pragma unroll
+    for (int i = 0; i < DPL; ++i) {
+      const int d = kg + 4 * i;
+      if (d < D) state[sbase + (long)d * DV + c] = S[i];
+    }
+  }
+}
+
+// Per (token, head): out = rmsnorm_DV(o) * w * silu(gate), rounded to T.
+// One wave per head, lanes over value channels.
+template <typename T>
+__global__ __launch_bounds__(256) void gla_out_norm_gate_kernel(
+    T* __restrict__ out, long out_stride, const float* __restrict__ o,
+    const T* __restrict__ weight, const T* __restrict__ gate, long g_stride,
+    int H, int DV, float eps) {
+  const long tok = blockIdx.x;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  for (int h = w; h < H; h += 4) {
+    const float* oh = o + (tok * H + h) * DV;
+    float ss = 0.f;
+    for (int c = lane; c < DV; c += 64) ss += oh[c] * oh[c];
+    ss = wave_reduce_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / DV + eps);
+    for (int c = lane; c < DV; c += 64) {
+      const float gt = to_f32(gate[tok * g_stride + (long)h * DV + c]);
+      const float sg = gt / (1.0f + expf(-gt));
+      out[tok * out_stride + (long)h * DV + c] =
+          from_f32<T>(oh[c] * inv * to_f32(weight[c]) * sg);
+    }
+  }
+}

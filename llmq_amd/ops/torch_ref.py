@@ -239,3 +239,141 @@ def sample_tokens(
         probs = torch.softmax(l, dim=-1)
         out[i] = torch.multinomial(probs, 1, generator=generator).squeeze(0)
     return out
+
+
+# ----------------------------------------------------- hybrid decoders ----
+# Reference forms of the hybrid-decoder ops (fp32 residual stream, block-
+# local biased attention over the paged cache, gated-linear-attention
+# recurrence over state slots). Same contracts as the HIP kernels.
+
+
+def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
+                 out_dtype: torch.dtype) -> torch.Tensor:
+    xf = x.float()
+    inv = 1.0 / torch.sqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
+    return (xf * inv * (weight.float() + offset)).to(out_dtype)
+
+
+def sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset):
+    """residual(fp32) += rmsnorm(x)*(w_post+offset); returns
+    rmsnorm(residual)*(w_pre+offset) in x's dtype. residual updated in place."""
+    residual.add_(rmsnorm_cast(x, w_post, eps, offset, torch.float32))
+    return rmsnorm_cast(residual, w_pre, eps, offset, x.dtype)
+
+
+def act_and_mul(x: torch.Tensor, gelu: bool) -> torch.Tensor:
+    return gelu_tanh_and_mul(x) if gelu else silu_and_mul(x)
+
+
+def qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, lam, k_cache, v_cache, slots, eps):
+    """q [T, nq] normalised in place over its whole width; k normalised and
+    v (blended with v_first when given) scattered into the paged cache."""
+    q.copy_(rmsnorm_cast(q, q_w, eps, 0.0, q.dtype))
+    kn = rmsnorm_cast(k, k_w, eps, 0.0, k.dtype)
+    vv = v.float()
+    if v_first is not None:
+        vv = (1.0 - lam) * vv + lam * v_first.float()
+    G, bs, D = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    DV = v_cache.shape[3]
+    keep = slots >= 0
+    s = slots[keep].long()
+    k_cache[s // bs, :, s % bs, :] = kn[keep].view(-1, G, D).to(k_cache.dtype)
+    v_cache[s // bs, :, s % bs, :] = vv[keep].view(-1, G, DV).to(v_cache.dtype)
+
+
+def _block_local_attend(qb, kc, vc, bias, pos, span, scale, gate):
+    """qb [n, H, D] at absolute positions pos [n]; kc [L, G, D], vc [L, G, DV]
+    the sequence's cached keys/values for positions 0..L-1."""
+    n, H, _ = qb.shape
+    G = kc.shape[1]
+    lo = int(pos[0]) // span * span
+    kk = kc[lo:].float().repeat_interleave(H // G, dim=1)
+    vv = vc[lo:].float().repeat_interleave(H // G, dim=1)
+    j = torch.arange(lo, kc.shape[0], device=qb.device).view(1, -1)
+    i = pos.view(-1, 1)
+    vis = (j <= i) & (j // span == i // span)
+    dist = (i - j).clamp_(0, bias.shape[0] - 1)
+    scores = torch.einsum("ihd,jhd->hij", qb.float(), kk) * scale
+    scores = scores + bias[dist].permute(2, 0, 1)
+    scores = scores.masked_fill(~vis.unsqueeze(0), float("-inf"))
+    out = torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), vv)
+    if gate is not None:
+        out = out * torch.sigmoid(gate.float()).unsqueeze(-1)
+    return out
+
+
+def _gather_seq(cache, table, length):
+    bs = cache.shape[2]
+    nb = (length + bs - 1) // bs
+    blocks = table[:nb].long()
+    return cache[blocks].permute(0, 2, 1, 3).reshape(nb * bs, cache.shape[1], cache.shape[3])[:length]
+
+
+def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q, q_start,
+                            span, scale):
+    T, H, _ = q.shape
+    out = q.new_empty(T, H, v_cache.shape[3])
+    for b in range(len(q_start)):
+        s, e = int(cu_q[b]), int(cu_q[b + 1])
+        if e == s:
+            continue
+        p0 = int(q_start[b])
+        L = p0 + (e - s)
+        kc = _gather_seq(k_cache, block_tables[b], L)
+        vc = _gather_seq(v_cache, block_tables[b], L)
+        pos = torch.arange(p0, L, device=q.device)
+        # rows of one portion may straddle several spans: attend span by span
+        start = 0
+        while start < e - s:
+            first = p0 + start
+            stop = min(e - s, start + (span - first % span))
+            rows = slice(s + start, s + stop)
+            out[rows] = _block_local_attend(
+                q[rows], kc[: p0 + stop], vc[: p0 + stop], bias, pos[start:stop], span, scale,
+                None if gate is None else gate[rows],
+            ).to(q.dtype)
+            start = stop
+    return out
+
+
+def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, context_lens,
+                           span, scale):
+    B, H, _ = q.shape
+    out = q.new_empty(B, H, v_cache.shape[3])
+    for b in range(B):
+        L = int(context_lens[b])
+        kc = _gather_seq(k_cache, block_tables[b], L)
+        vc = _gather_seq(v_cache, block_tables[b], L)
+        pos = torch.tensor([L - 1], device=q.device)
+        out[b : b + 1] = _block_local_attend(
+            q[b : b + 1], kc, vc, bias, pos, span, scale,
+            None if gate is None else gate[b : b + 1],
+        ).to(q.dtype)
+    return out
+
+
+def gla_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau):
+    """q,k,z [T,H,D], v [T,H,DV] → o [T,H,DV] fp32; state [slots,H,D,DV] fp32
+    advanced in place (zero start where fresh)."""
+    T, H, D = q.shape
+    o = torch.empty(T, H, v.shape[2], dtype=torch.float32, device=q.device)
+    zf = z.float() + z_bias.view(1, H, D)
+    alpha = torch.exp(torch.nn.functional.logsigmoid(zf) / tau)
+    qf = q.float() * (1.0 / (D ** 0.5))
+    kf, vf = k.float(), v.float()
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        S = torch.zeros_like(state[slot]) if int(fresh[b]) else state[slot].clone()
+        for t in range(s, e):
+            S = alpha[t].unsqueeze(-1) * S + kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    return o
+
+
+def gla_out_norm_gate(o, weight, gate, eps, out_dtype):
+    T, H, DV = o.shape
+    y = o * (1.0 / torch.sqrt(o.pow(2).mean(dim=-1, keepdim=True) + eps)) * weight.float()
+    y = y.reshape(T, H * DV) * torch.nn.functional.silu(gate.float())
+    return y.to(out_dtype)
