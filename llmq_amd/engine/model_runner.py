@@ -66,6 +66,7 @@ class ModelRunner:
         # decode path, "prefill" for the prefill segment of an OVERLAPPED
         # split mixed step — two concurrent streams must not share them).
         self._sample_bufs: Dict[str, Dict[str, torch.Tensor]] = {}
+        self._staging_done = None  # event: last step's pinned→device copies landed
         # Models whose prompt-portion attention reads the paged cache through
         # the block table (no gathered K/V copy), and models with recurrent
         # layers (per-sequence state slots), get the extra step metadata.
@@ -399,6 +400,12 @@ class ModelRunner:
         self, seqs: List[Sequence], bucket: int, ids, pos, slots, ctx, want=None
     ) -> torch.Tensor:
         B = len(seqs)
+        # The pinned staging buffers are rewritten every step: the previous
+        # step's async copies out of them must have landed first. Sampling
+        # steps synchronise anyway (tokens go to the host); a replay step
+        # that wants no logits does not.
+        if self._staging_done is not None:
+            self._staging_done.synchronize()
         # Stage metadata through pinned host buffers, one async copy each.
         self.h_ids[:B] = torch.tensor(ids, dtype=torch.long)
         self.h_pos[:B] = torch.tensor(pos, dtype=torch.long)
@@ -445,6 +452,9 @@ class ModelRunner:
             self.h_rec_fresh[B:bucket] = 1
             self.in_rec.slots[:bucket].copy_(self.h_rec_slots[:bucket], non_blocking=True)
             self.in_rec.fresh[:bucket].copy_(self.h_rec_fresh[:bucket], non_blocking=True)
+        if self._staging_done is None:
+            self._staging_done = torch.cuda.Event()
+        self._staging_done.record()
         self._graphs[bucket].replay()
         if want is not None:
             return self._logits_at(self.out_hidden[:B], [b for b, ws in enumerate(want) if ws])
