@@ -40,12 +40,10 @@ def distance_bias(T: int, table: torch.Tensor, far: float) -> torch.Tensor:
     """[H, T, T] additive bias, entry (h, i, j) = table[bucket(i - j), h]
     for j <= i (0 above the diagonal, masked anyway)."""
     rows, H = table.shape
-    out = torch.zeros(H, T, T, dtype=table.dtype)
     per_dist = torch.stack([table[distance_bucket(n, rows, far)] for n in range(T)])  # [T, H]
-    for i in range(T):
-        for j in range(i + 1):
-            out[:, i, j] = per_dist[i - j]
-    return out
+    i = torch.arange(T).view(-1, 1)
+    j = torch.arange(T).view(1, -1)
+    return per_dist[(i - j).clamp(min=0)].permute(2, 0, 1).contiguous()
 
 
 def block_causal_mask(T: int, size: int) -> torch.Tensor:
@@ -147,3 +145,11 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int],
     if return_layers:
         return logits, torch.stack(per_layer)
     return logits
+
+
+def greedy(config: dict, tensors: Dict[str, torch.Tensor], prompt: List[int], n: int) -> List[int]:
+    """n greedy tokens after the prompt, recomputing the whole sequence each time."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(config, tensors, toks)[-1].argmax()))
+    return toks[len(prompt):]
