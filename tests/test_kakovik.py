@@ -121,14 +121,19 @@ def make_engine(path, target, blocks=64, block_size=16, max_seqs=4, prefill_budg
 
 
 def tolerance(target):
-    return 3e-2 if target[1] == "bfloat16" else 2e-4
+    """(worst row, mean over rows) of the relative rms error. fp32 is the
+    sharp comparison; bf16 rounds every GEMM input and output of a six-layer
+    stack and only has to stay at rounding level."""
+    return (8e-2, 2.5e-2) if target[1] == "bfloat16" else (2e-4, 5e-5)
 
 
 def assert_close(got, want, target, what=""):
     got, want = got.double().cpu(), want.double()
     err = (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt()
-    worst = float(err.max())
-    assert worst < tolerance(target), f"{what}: worst row error {worst:.3e} at row {int(err.argmax())}"
+    worst, mean = float(err.max()), float(err.mean())
+    lim_worst, lim_mean = tolerance(target)
+    assert worst < lim_worst, f"{what}: worst row error {worst:.3e} at row {int(err.argmax())}"
+    assert mean < lim_mean, f"{what}: mean row error {mean:.3e}"
 
 
 def replay(engine, rid, toks, cuts, end=True):
