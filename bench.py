@@ -28,6 +28,78 @@ import sys
 import time
 
 
+def compare_hybrid(args) -> None:
+    """Prefill and decode throughput, one engine per model, same workload:
+    --batch sequences of --prompt-len random tokens prefilled in budgeted
+    steps (timed), then --steps hipGraph decode steps of the full batch
+    (timed after --warmup). Random-init bf16 weights, one GPU."""
+    import numpy as np
+    import torch
+
+    from llmq_amd.engine.config import EngineConfig
+    from llmq_amd.engine.engine import LLMEngine
+    from llmq_amd.engine.sampling_params import SamplingParams
+
+    use_gpu = torch.cuda.is_available()
+    models = args.compare_models.split(",")
+    batch, prompt_len = min(args.batch, 64), args.prompt_len
+    if not use_gpu:
+        models, batch, prompt_len = ["tiny-kakovik", "tiny-llama"], 4, 48
+    for name in models:
+        engine = LLMEngine(EngineConfig(
+            model=name, max_num_seqs=batch,
+            max_model_len=(prompt_len + args.steps + args.warmup + 64) if use_gpu else 256,
+            max_prefill_tokens=16384, load_weights=False, fast_init=True,
+            enforce_eager=args.eager, hipgraph_max_batch=batch, seed=1234,
+        ))
+        rng = np.random.default_rng(7)
+        params = SamplingParams(temperature=args.temperature, max_tokens=1 << 20, ignore_eos=True)
+
+        def sync():
+            if use_gpu:
+                torch.cuda.synchronize()
+
+        def load(tag):
+            for i in range(batch):
+                ids = rng.integers(0, engine.spec.vocab_size, size=prompt_len).tolist()
+                engine.add_request(f"{tag}-{i}", prompt_token_ids=ids, params=params)
+
+        def prefill_all():
+            while engine.scheduler.num_waiting > 0 or engine.scheduler.prefilling:
+                engine.step()
+            sync()
+
+        load("warm")            # untimed pass: allocator, GEMM selection
+        prefill_all()
+        for i in range(batch):
+            engine.abort_request(f"warm-{i}")
+        load("run")
+        sync()
+        t0 = time.perf_counter()
+        prefill_all()
+        prefill_s = time.perf_counter() - t0
+        for _ in range(args.warmup):
+            engine.step()
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            engine.step()
+        sync()
+        decode_s = time.perf_counter() - t0
+        print(json.dumps({
+            "model": name, "family": engine.spec.family,
+            "params_b": round(engine.spec.param_count() / 1e9, 3),
+            "batch": batch, "prompt_len": prompt_len,
+            "prefill_tokens_per_sec": round(batch * prompt_len / prefill_s, 1),
+            "decode_tokens_per_sec": round(batch * args.steps / decode_s, 1),
+            "decode_ms_per_step": round(decode_s / args.steps * 1000.0, 3),
+            "dtype": "bf16" if use_gpu else "fp32", "data": "synthetic",
+        }), flush=True)
+        del engine
+        if use_gpu:
+            torch.cuda.empty_cache()
+
+
 def main() -> None:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -49,7 +121,15 @@ def main() -> None:
                         "model sharded over RCCL/xGMI (BASELINE config #4, "
                         "e.g. --tp 8 --model tower-plus-72b under torchrun "
                         "--nproc-per-node 8). Default 0 = data-parallel.")
+    parser.add_argument("--compare-hybrid", action="store_true",
+                        help="instead of the headline workload: prefill and decode "
+                        "throughput of the Kakovik hybrid presets beside the Llama "
+                        "presets of equal layer sizes (one JSON line per model)")
+    parser.add_argument("--compare-models", default="kakovik-1b,llama-3.2-1b,kakovik-3b,llama-3.2-3b")
     args = parser.parse_args()
+    if args.compare_hybrid:
+        compare_hybrid(args)
+        return
 
     import torch
 

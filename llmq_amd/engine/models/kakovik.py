@@ -24,7 +24,7 @@ MI355X mapping, in the manner of the other families:
   advanced by one kernel for any mix of portions and single tokens.
 
 The per-distance bias is tabulated once per layer for distances inside one
-span (bias[n, h], n < span) — the kernels index it by i - j.
+span (bias[h, n], n < span) — the kernels index it by i - j.
 """
 
 from __future__ import annotations
@@ -54,7 +54,7 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
 class HybridLayerWeights:
     def __init__(self) -> None:
         self.t: Dict[str, torch.Tensor] = {}   # checkpoint-shaped tensors
-        self.bias: Optional[torch.Tensor] = None   # [span, H] fp32 (attention)
+        self.bias: Optional[torch.Tensor] = None   # [H, span] fp32 (attention)
         self.lam: float = 0.0                      # value-blend weight
         self.mixes: bool = False                   # blends with v_first
         self.provides_v_first: bool = False
@@ -118,7 +118,10 @@ class KakovikLM:
                 nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
                 if m.heads % m.kv_heads:
                     raise ValueError("heads must be a multiple of kv_heads")
-                t["qkvg"] = self._empty(nq + nk + nv + m.heads, W)
+                # rows padded to a multiple of 8: row strides of the GEMM
+                # output stay 16-byte aligned for the vector loads of q
+                t["qkvg"] = self._empty(-(-(nq + nk + nv + m.heads) // 8) * 8, W)
+                t["qkvg"].zero_()
                 t["q_norm"], t["k_norm"] = self._empty(nq), self._empty(nk)
                 t["rel"] = self._empty(m.bias_rows, m.heads)
                 t["vmix"] = self._empty(())
@@ -151,7 +154,7 @@ class KakovikLM:
                 continue
             rel = lw.t["rel"].float().cpu()
             rows = [distance_bucket(n, m.bias_rows, m.bias_far) for n in range(m.span)]
-            lw.bias = rel[torch.tensor(rows, dtype=torch.long)].contiguous().to(self.device)
+            lw.bias = rel[torch.tensor(rows, dtype=torch.long)].t().contiguous().to(self.device)
             lw.lam = float(lw.t["vmix"].float().item())
             if m.v_mix:
                 nv = m.kv_heads * m.vdim
@@ -211,7 +214,7 @@ class KakovikLM:
         nq, nk, nv = m.heads * m.dim, m.kv_heads * m.dim, m.kv_heads * m.vdim
         p = F.linear(h, lw.t["qkvg"])
         q, k, v = p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv]
-        gate = p[:, nq + nk + nv:]
+        gate = p[:, nq + nk + nv:nq + nk + nv + m.heads]
         kc, vc = kv_cache.k[i], kv_cache.v[i]
         ops.qknorm_vmix_cache(
             q, k, v, lw.t["q_norm"], lw.t["k_norm"],

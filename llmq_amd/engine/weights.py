@@ -133,8 +133,9 @@ def load_kakovik_weights(model, path: Path) -> None:
         copy_(t["norm1b"], get(p + "norm1b"))
         mx = p + "mix."
         if ls.mixer.kind == "attention":
-            copy_(t["qkvg"], torch.cat([get(mx + "q"), get(mx + "k"), get(mx + "v"),
-                                        get(mx + "g")], dim=0))
+            packed = torch.cat([get(mx + "q"), get(mx + "k"), get(mx + "v"), get(mx + "g")], dim=0)
+            t["qkvg"].zero_()  # trailing alignment rows
+            copy_(t["qkvg"][: packed.shape[0]], packed)
             copy_(t["q_norm"], get(mx + "q.norm"))
             copy_(t["k_norm"], get(mx + "k.norm"))
             copy_(t["rel"], get(mx + "rel"))

@@ -165,8 +165,8 @@ AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optio
   TORCH_CHECK(a.H % a.G == 0, "heads must be a multiple of kv heads");
   TORCH_CHECK(a.DV <= 256, "value size above 256 is not supported");
   TORCH_CHECK(span >= 1 && bias.scalar_type() == at::kFloat && bias.is_contiguous() &&
-              bias.dim() == 2 && bias.size(0) >= span && bias.size(1) == a.H,
-              "bias must be fp32 [span, H]");
+              bias.dim() == 2 && bias.size(0) == a.H && bias.size(1) == span,
+              "bias must be fp32 [H, span]");
   TORCH_CHECK(q.scalar_type() == out.scalar_type() && q.scalar_type() == k_cache.scalar_type() &&
               q.scalar_type() == v_cache.scalar_type());
   HY_I32(block_tables);
@@ -194,6 +194,38 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
   HY_I32(cu_q); HY_I32(q_start);
   const int B = q_start.numel();
   TORCH_CHECK(cu_q.numel() == B + 1 && block_tables.size(0) == B && max_q >= 1);
+  // bf16 with 16-byte-aligned q rows and key rows: the matrix-core kernel
+  // (LLMQ_HYBRID_ATTN_VALU=1 keeps the fp32-ALU kernel, for A/B runs)
+  static const bool force_valu = [] {
+    const char* e = getenv("LLMQ_HYBRID_ATTN_VALU");
+    return e && e[0] == '1';
+  }();
+  if (q.scalar_type() == at::kBFloat16 && !force_valu && a.D % 8 == 0 && a.D <= 256 &&
+      q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
+    const int ksn = (a.D + 31) / 32, dtn = (a.DV + 15) / 16;
+    const size_t lds = sizeof(short) * ((size_t)kMfmaKT * (ksn * 32 + 8) +
+                                        (size_t)dtn * 16 * kMfmaKP + (size_t)4 * 2 * 16 * kMfmaKP);
+    const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H, B);
+    using bf = __hip_bfloat16;
+    auto launch = [&]<int KS, int DT>() {
+      auto kern = chunk_bias_attn_prefill_mfma_kernel<KS, DT>;
+      allow_lds(kern, lds);
+      hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(),
+                         reinterpret_cast<bf*>(out.data_ptr()), out.stride(0),
+                         reinterpret_cast<const bf*>(q.data_ptr()), q.stride(0),
+                         gate.has_value() ? reinterpret_cast<const bf*>(gate->data_ptr()) : nullptr,
+                         gate.has_value() ? gate->stride(0) : 0L,
+                         reinterpret_cast<const bf*>(k_cache.data_ptr()),
+                         reinterpret_cast<const bf*>(v_cache.data_ptr()), bias.data_ptr<float>(),
+                         block_tables.data_ptr<int>(), (int)block_tables.stride(0),
+                         cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
+                         (int)span, (float)scale);
+    };
+    if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
+    else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
+    else launch.template operator()<8, 16>();
+    return;
+  }
   const size_t lds = sizeof(float) * ((size_t)kAttnKT * (a.D + 1) + (size_t)kAttnKT * a.DV +
                                       (size_t)kAttnQT * a.D + (size_t)kAttnQT * kAttnKT);
   const dim3 grid((max_q + kAttnQT - 1) / kAttnQT, a.H, B);

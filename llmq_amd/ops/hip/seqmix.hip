@@ -165,7 +165,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     const T* __restrict__ q, long q_stride,
     const T* __restrict__ gate, long g_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const float* __restrict__ bias,        // [span, H]
+    const float* __restrict__ bias,        // [H, span]
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q,          // [B+1]
     const int* __restrict__ q_start,       // [B] position of a sequence's first query
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const int i = pos0 + w * 4 + r;
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
                        key / span == i / span;
-      const float sc = vis ? s[r] + bias[(long)(i - key) * H + h] : -INFINITY;
+      const float sc = vis ? s[r] + bias[(long)h * span + (i - key)] : -INFINITY;
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -292,6 +292,211 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
   }
 }
 
+// The bf16 form of the same kernel on the matrix cores.
+//
+// Workgroup = 64 query rows x 1 head, one wave per 16 rows. Per 64-key tile:
+// K is staged row-major [key][D] and V transposed [channel][key] in LDS, so
+// every MFMA operand is one 16-byte LDS read. S = Q K^T and O += P V run on
+// v_mfma_f32_16x16x32_bf16 (A: row = lane%16, k = 8*(lane/16)..+7; C: rows
+// 4*(lane/16)+reg, column lane%16), which puts a query row's scores and its
+// output in the same registers of the same lanes: the online-softmax rescale
+// needs no exchange. Scores, bias, mask and softmax stay fp32. The weights
+// enter the second product as TWO bf16 planes (p = hi + lo, lo the rounding
+// remainder of hi), so the product sees them to 16 mantissa bits instead of 8.
+typedef __attribute__((ext_vector_type(8))) short sm_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float sm_f32x4;
+constexpr int kMfmaQT = 64;
+constexpr int kMfmaKT = 64;
+constexpr int kMfmaKP = kMfmaKT + 8;   // padded key stride of the V^T and P tiles
+
+template <int KS, int DT>
+__global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
+    __hip_bfloat16* __restrict__ out, long out_stride,
+    const __hip_bfloat16* __restrict__ q, long q_stride,
+    const __hip_bfloat16* __restrict__ gate, long g_stride,
+    const __hip_bfloat16* __restrict__ k_cache, const __hip_bfloat16* __restrict__ v_cache,
+    const float* __restrict__ bias,        // [H, span]
+    const int* __restrict__ block_tables, int bt_stride,
+    const int* __restrict__ cu_q, const int* __restrict__ q_start,
+    int H, int G, int D, int DV, int block_size, int span, float scale) {
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  const int b = blockIdx.z, h = blockIdx.y;
+  const int row0 = cu_q[b];
+  const int nq = cu_q[b + 1] - row0;
+  const int r0 = blockIdx.x * kMfmaQT;
+  if (r0 >= nq) return;
+  const int rows = min(kMfmaQT, nq - r0);
+  const int pos0 = q_start[b] + r0;
+  const int pos_last = pos0 + rows - 1;
+  const int g = h / (H / G);
+  const int ksn = (D + 31) / 32, dtn = (DV + 15) / 16;
+  const int Dp = ksn * 32, DS = Dp + 8;
+  short* Ks = reinterpret_cast<short*>(smem_raw);     // [KT][DS]
+  short* Vt = Ks + kMfmaKT * DS;                      // [dtn*16][KP]
+  short* Ps = Vt + dtn * 16 * kMfmaKP;                // [4 waves][hi, lo][16][KP]
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int col = lane & 15, kgrp = lane >> 4;
+
+  sm_bf16x8 qf[KS];
+  {
+    const int r = w * 16 + col;
+    const __hip_bfloat16* qr = q + (long)(row0 + r0 + r) * q_stride + (long)h * D;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d8 = ks * 32 + kgrp * 8;
+      qf[ks] = (r < rows && d8 < D) ? *reinterpret_cast<const sm_bf16x8*>(qr + d8)
+                                    : sm_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    }
+  }
+  int irow[4], lorow[4];
+  float m[4], l[4];
+#pragma unroll
+  for (int reg = 0; reg < 4; ++reg) {
+    const int r = w * 16 + kgrp * 4 + reg;
+    irow[reg] = r < rows ? pos0 + r : -1;       // -1: no key satisfies key <= irow
+    lorow[reg] = r < rows ? ((pos0 + r) / span) * span : 0;
+    m[reg] = -INFINITY;
+    l[reg] = 0.f;
+  }
+  sm_f32x4 o[DT];
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) o[dt] = sm_f32x4{0.f, 0.f, 0.f, 0.f};
+  const int wave_first = pos0 + w * 16;
+  const int wave_last = min(pos_last, wave_first + 15);
+  const int wave_lo = (wave_first / span) * span;
+  const bool wave_rows = w * 16 < rows;
+  const int* bt = block_tables + (long)b * bt_stride;
+  const float* bias_h = bias + (long)h * span;
+  short* Pw = Ps + w * 2 * 16 * kMfmaKP;
+  const int kgran = Dp / 8, vgran = dtn * 2;
+  const bool v_vec = (DV % 8) == 0;
+
+  for (int kt = (pos0 / span) * span; kt <= pos_last; kt += kMfmaKT) {
+    __syncthreads();
+    for (int idx = tid; idx < kMfmaKT * kgran; idx += 256) {
+      const int key = idx / kgran, d8 = (idx % kgran) * 8;
+      const int gkey = kt + key;
+      sm_bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (gkey <= pos_last && d8 < D) {
+        const long base = ((long)bt[gkey / block_size] * G + g) * block_size + gkey % block_size;
+        val = *reinterpret_cast<const sm_bf16x8*>(k_cache + base * D + d8);
+      }
+      *reinterpret_cast<sm_bf16x8*>(Ks + key * DS + d8) = val;
+    }
+    for (int idx = tid; idx < kMfmaKT * vgran; idx += 256) {
+      const int key = idx % kMfmaKT, d8 = (idx / kMfmaKT) * 8;
+      const int gkey = kt + key;
+      short e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (gkey <= pos_last && d8 < DV) {
+        const long base = ((long)bt[gkey / block_size] * G + g) * block_size + gkey % block_size;
+        const __hip_bfloat16* vr = v_cache + base * DV + d8;
+        if (v_vec) {
+          *reinterpret_cast<sm_bf16x8*>(e) = *reinterpret_cast<const sm_bf16x8*>(vr);
+        } else {
+          for (int j = 0; j < 8; ++j)
+            if (d8 + j < DV) e[j] = __bfloat16_as_short(vr[j]);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Vt[(d8 + j) * kMfmaKP + key] = e[j];
+    }
+    __syncthreads();
+    const bool active = wave_rows && kt <= wave_last && kt + kMfmaKT - 1 >= wave_lo;
+    if (active) {
+      sm_f32x4 s[4];
+#pragma unroll
+      for (int ct = 0; ct < 4; ++ct) {
+        s[ct] = sm_f32x4{0.f, 0.f, 0.f, 0.f};
+        const short* kr = Ks + (ct * 16 + col) * DS + kgrp * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          if (ks < ksn) {
+            const sm_bf16x8 bf = *reinterpret_cast<const sm_bf16x8*>(kr + ks * 32);
+            s[ct] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[ks], bf, s[ct], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int reg = 0; reg < 4; ++reg) {
+        float sv[4], tmax = -INFINITY;
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          const int key = kt + ct * 16 + col;
+          const bool vis = key >= lorow[reg] && key <= irow[reg];
+          sv[ct] = vis ? s[ct][reg] * scale + bias_h[irow[reg] - key] : -INFINITY;
+          tmax = fmaxf(tmax, sv[ct]);
+        }
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 1, WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 2, WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 4, WAVE));
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 8, WAVE));
+        const float m_new = fmaxf(m[reg], tmax);
+        float alpha = 1.f, psum = 0.f;
+        float pv[4] = {0.f, 0.f, 0.f, 0.f};
+        if (m_new > -INFINITY) {
+          alpha = __expf(m[reg] - m_new);
+#pragma unroll
+          for (int ct = 0; ct < 4; ++ct) {
+            pv[ct] = sv[ct] > -INFINITY ? __expf(sv[ct] - m_new) : 0.f;
+            psum += pv[ct];
+          }
+        }
+        l[reg] = l[reg] * alpha + psum;   // per-lane partial; reduced at the end
+        m[reg] = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) o[dt][reg] *= alpha;
+        short* pr = Pw + (kgrp * 4 + reg) * kMfmaKP + col;
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+          const __hip_bfloat16 hi = __float2bfloat16(pv[ct]);
+          const __hip_bfloat16 lo = __float2bfloat16(pv[ct] - __bfloat162float(hi));
+          pr[ct * 16] = __bfloat16_as_short(hi);
+          pr[16 * kMfmaKP + ct * 16] = __bfloat16_as_short(lo);
+        }
+      }
+    }
+    __syncthreads();
+    if (active) {
+#pragma unroll
+      for (int k2 = 0; k2 < kMfmaKT / 32; ++k2) {
+        const sm_bf16x8 a_hi = *reinterpret_cast<const sm_bf16x8*>(
+            Pw + col * kMfmaKP + k2 * 32 + kgrp * 8);
+        const sm_bf16x8 a_lo = *reinterpret_cast<const sm_bf16x8*>(
+            Pw + (16 + col) * kMfmaKP + k2 * 32 + kgrp * 8);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+          if (dt < dtn) {
+            const sm_bf16x8 bf = *reinterpret_cast<const sm_bf16x8*>(
+                Vt + (dt * 16 + col) * kMfmaKP + k2 * 32 + kgrp * 8);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_hi, bf, o[dt], 0, 0, 0);
+            o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a_lo, bf, o[dt], 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int reg = 0; reg < 4; ++reg) {
+    float ll = l[reg];
+    ll += __shfl_xor(ll, 1, WAVE);
+    ll += __shfl_xor(ll, 2, WAVE);
+    ll += __shfl_xor(ll, 4, WAVE);
+    ll += __shfl_xor(ll, 8, WAVE);
+    const int r = w * 16 + kgrp * 4 + reg;
+    if (r >= rows) continue;
+    const long trow = row0 + r0 + r;
+    float gs = 1.f;
+    if (gate) gs = 1.0f / (1.0f + expf(-__bfloat162float(gate[trow * g_stride + h])));
+    const float inv = gs / ll;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int c = dt * 16 + col;
+      if (dt < dtn && c < DV)
+        out[trow * out_stride + (long)h * DV + c] = __float2bfloat16(o[dt][reg] * inv);
+    }
+  }
+}
+
 // ------------------------------------------------ attention: single tokens --
 // One workgroup per (sequence, head); the query is the sequence's newest
 // token (position ctx-1). Waves take key tiles of 64 round-robin, each with
@@ -333,7 +538,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
       const T* kr = k_cache + base * D;
       float s = 0.f;
       for (int d = 0; d < D; ++d) s += Qs[d] * to_f32(kr[d]);
-      sc = s + bias[(long)(i - key) * H + h];
+      sc = s + bias[(long)h * span + (i - key)];
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));  // nk >= 1: finite
     const float corr = expf(m - m_new);

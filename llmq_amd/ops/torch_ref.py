@@ -292,9 +292,9 @@ def _block_local_attend(qb, kc, vc, bias, pos, span, scale, gate):
     j = torch.arange(lo, kc.shape[0], device=qb.device).view(1, -1)
     i = pos.view(-1, 1)
     vis = (j <= i) & (j // span == i // span)
-    dist = (i - j).clamp_(0, bias.shape[0] - 1)
+    dist = (i - j).clamp_(0, bias.shape[1] - 1)
     scores = torch.einsum("ihd,jhd->hij", qb.float(), kk) * scale
-    scores = scores + bias[dist].permute(2, 0, 1)
+    scores = scores + bias[:, dist]
     scores = scores.masked_fill(~vis.unsqueeze(0), float("-inf"))
     out = torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), vv)
     if gate is not None:

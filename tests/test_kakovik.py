@@ -336,7 +336,7 @@ def _needle_case(device, dtype, span, key_pos, query_pos, decode, block_size=16)
     b, o = int(table[0, key_pos // block_size]), key_pos % block_size
     kc[b, 0, o, 0] = 40.0
     vc[b, 0, o, :] = -3.0
-    bias = torch.zeros(span, 1)
+    bias = torch.zeros(1, span)
     kc, vc, bias, table = kc.to(device), vc.to(device), bias.to(device), table.to(device)
     if decode:
         q = torch.zeros(1, 1, D, dtype=dtype, device=device)
@@ -386,12 +386,12 @@ def test_bias_moves_attention_by_distance(target):
     vc = torch.zeros(2, 1, bs, 16, dtype=dtype, device=device)
     for p in range(n):
         vc[1, 0, p, p] = 1.0                 # value p marks position p
-    bias = torch.linspace(-2, 2, span).view(span, 1).to(device)
+    bias = torch.linspace(-2, 2, span).view(1, span).to(device)
     table = torch.tensor([[1]], dtype=torch.int32, device=device)
     q = torch.zeros(1, 1, 8, dtype=dtype, device=device)
     out = ops.chunk_bias_attn_decode(q, None, kc, vc, bias, table,
                                      torch.tensor([n], dtype=torch.int32, device=device), span, 1.0)
-    want = torch.softmax(bias[:, 0].flip(0).double().cpu(), 0)  # key j at distance n-1-j
+    want = torch.softmax(bias[0].flip(0).double().cpu(), 0)  # key j at distance n-1-j
     assert_close(out[0, 0, :n].view(1, -1), want.view(1, -1), target)
 
 
