@@ -203,11 +203,13 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
   if (q.scalar_type() == at::kBFloat16 && !force_valu && a.D % 8 == 0 && a.D <= 256 &&
       q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
     const int ksn = (a.D + 31) / 32, dtn = (a.DV + 15) / 16;
-    const size_t lds = sizeof(short) * ((size_t)kMfmaKT * (ksn * 32 + 8) +
-                                        (size_t)dtn * 16 * kMfmaKP + (size_t)4 * 2 * 16 * kMfmaKP);
     const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H, B);
     using bf = __hip_bfloat16;
     auto launch = [&]<int KS, int DT>() {
+      // K tile, V^T tile (all DT*16 channel rows), P hi/lo per wave, bias slice
+      const size_t lds = sizeof(short) * ((size_t)kMfmaKT * (ksn * 32 + 8) +
+                                          (size_t)DT * 16 * kMfmaKP +
+                                          (size_t)4 * 2 * 16 * kMfmaKP) + 128 * sizeof(float);
       auto kern = chunk_bias_attn_prefill_mfma_kernel<KS, DT>;
       allow_lds(kern, lds);
       hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(),

@@ -310,7 +310,7 @@ constexpr int kMfmaKT = 64;
 constexpr int kMfmaKP = kMfmaKT + 8;   // padded key stride of the V^T and P tiles
 
 template <int KS, int DT>
-__global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
+__global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     __hip_bfloat16* __restrict__ out, long out_stride,
     const __hip_bfloat16* __restrict__ q, long q_stride,
     const __hip_bfloat16* __restrict__ gate, long g_stride,
@@ -320,6 +320,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
+  constexpr int VG = DT / 2;             // 32-channel groups of V per thread
   const int b = blockIdx.z, h = blockIdx.y;
   const int row0 = cu_q[b];
   const int nq = cu_q[b + 1] - row0;
@@ -332,8 +333,9 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
   const int ksn = (D + 31) / 32, dtn = (DV + 15) / 16;
   const int Dp = ksn * 32, DS = Dp + 8;
   short* Ks = reinterpret_cast<short*>(smem_raw);     // [KT][DS]
-  short* Vt = Ks + kMfmaKT * DS;                      // [dtn*16][KP]
-  short* Ps = Vt + dtn * 16 * kMfmaKP;                // [4 waves][hi, lo][16][KP]
+  short* Vt = Ks + kMfmaKT * DS;                      // [DT*16][KP]
+  short* Ps = Vt + DT * 16 * kMfmaKP;                 // [4 waves][hi, lo][16][KP]
+  float* Bs = reinterpret_cast<float*>(Ps + 4 * 2 * 16 * kMfmaKP);  // [128] bias slice
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int col = lane & 15, kgrp = lane >> 4;
 
@@ -368,39 +370,65 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
   const int* bt = block_tables + (long)b * bt_stride;
   const float* bias_h = bias + (long)h * span;
   short* Pw = Ps + w * 2 * 16 * kMfmaKP;
-  const int kgran = Dp / 8, vgran = dtn * 2;
   const bool v_vec = (DV % 8) == 0;
 
-  for (int kt = (pos0 / span) * span; kt <= pos_last; kt += kMfmaKT) {
-    __syncthreads();
-    for (int idx = tid; idx < kMfmaKT * kgran; idx += 256) {
-      const int key = idx / kgran, d8 = (idx % kgran) * 8;
-      const int gkey = kt + key;
-      sm_bf16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (gkey <= pos_last && d8 < D) {
-        const long base = ((long)bt[gkey / block_size] * G + g) * block_size + gkey % block_size;
-        val = *reinterpret_cast<const sm_bf16x8*>(k_cache + base * D + d8);
-      }
-      *reinterpret_cast<sm_bf16x8*>(Ks + key * DS + d8) = val;
+  // Staging map: thread = (key = tid/4, sub = tid%4) moves the 16-byte
+  // granules sub*8 + 32*i of its key's K row and V row. The next tile's
+  // granules are fetched into registers before the current tile's math and
+  // written to LDS after it, so HBM/L2 latency hides behind the MFMAs.
+  const int skey = tid >> 2, sub = tid & 3;
+  sm_bf16x8 kreg[KS], vreg[VG];
+  const sm_bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  auto fetch = [&](int kt) {
+    const int gkey = kt + skey;
+    const bool live = gkey <= pos_last;
+    long base = 0;
+    if (live) base = ((long)bt[gkey / block_size] * G + g) * block_size + gkey % block_size;
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      const int d8 = sub * 8 + 32 * i;
+      kreg[i] = (live && d8 < D) ? *reinterpret_cast<const sm_bf16x8*>(k_cache + base * D + d8)
+                                 : zero8;
     }
-    for (int idx = tid; idx < kMfmaKT * vgran; idx += 256) {
-      const int key = idx % kMfmaKT, d8 = (idx / kMfmaKT) * 8;
-      const int gkey = kt + key;
-      short e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (gkey <= pos_last && d8 < DV) {
-        const long base = ((long)bt[gkey / block_size] * G + g) * block_size + gkey % block_size;
+#pragma unroll
+    for (int i = 0; i < VG; ++i) {
+      const int d8 = sub * 8 + 32 * i;
+      sm_bf16x8 e = zero8;
+      if (live && d8 < DV) {
         const __hip_bfloat16* vr = v_cache + base * DV + d8;
         if (v_vec) {
-          *reinterpret_cast<sm_bf16x8*>(e) = *reinterpret_cast<const sm_bf16x8*>(vr);
+          e = *reinterpret_cast<const sm_bf16x8*>(vr);
         } else {
+#pragma unroll
           for (int j = 0; j < 8; ++j)
             if (d8 + j < DV) e[j] = __bfloat16_as_short(vr[j]);
         }
       }
+      vreg[i] = e;
+    }
+  };
+  const int kt0 = (pos0 / span) * span;
+  fetch(kt0);
+  for (int kt = kt0; kt <= pos_last; kt += kMfmaKT) {
+    __syncthreads();
 #pragma unroll
-      for (int j = 0; j < 8; ++j) Vt[(d8 + j) * kMfmaKP + key] = e[j];
+    for (int i = 0; i < KS; ++i) {
+      const int d8 = sub * 8 + 32 * i;
+      if (d8 < Dp) *reinterpret_cast<sm_bf16x8*>(Ks + skey * DS + d8) = kreg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VG; ++i) {
+      const int d8 = sub * 8 + 32 * i;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) Vt[(d8 + j) * kMfmaKP + skey] = vreg[i][j];
+    }
+    if (tid < 127) {
+      // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)
+      const int d = pos0 - kt - 63 + tid;
+      Bs[tid] = (d >= 0 && d < span) ? bias_h[d] : 0.f;
     }
     __syncthreads();
+    if (kt + kMfmaKT <= pos_last) fetch(kt + kMfmaKT);
     const bool active = wave_rows && kt <= wave_last && kt + kMfmaKT - 1 >= wave_lo;
     if (active) {
       sm_f32x4 s[4];
@@ -419,11 +447,12 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_mfma_kernel(
 #pragma unroll
       for (int reg = 0; reg < 4; ++reg) {
         float sv[4], tmax = -INFINITY;
+        const float* brow = Bs + (w * 16 + kgrp * 4 + reg) + 63 - col;
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
           const int key = kt + ct * 16 + col;
           const bool vis = key >= lorow[reg] && key <= irow[reg];
-          sv[ct] = vis ? s[ct][reg] * scale + bias_h[irow[reg] - key] : -INFINITY;
+          sv[ct] = vis ? s[ct][reg] * scale + brow[-ct * 16] : -INFINITY;
           tmax = fmaxf(tmax, sv[ct]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 1, WAVE));
