@@ -67,6 +67,20 @@ void sandwich_norm_res32(at::Tensor x, at::Tensor residual, at::Tensor w_post, a
   TORCH_CHECK(w_post.scalar_type() == x.scalar_type() && w_pre.scalar_type() == x.scalar_type());
   const long rows = x.numel() / hidden;
   if (rows == 0) return;
+  if (x.scalar_type() == at::kBFloat16 && hidden % 8 == 0 && hidden <= 4 * 2048) {
+    using bf = __hip_bfloat16;
+    auto launch = [&]<int CH>() {
+      hipLaunchKernelGGL(sandwich_norm_res32_vec_kernel<CH>, dim3(rows), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<bf*>(x.data_ptr()), residual.data_ptr<float>(),
+                         reinterpret_cast<const bf*>(w_post.data_ptr()),
+                         reinterpret_cast<const bf*>(w_pre.data_ptr()), hidden, (float)eps,
+                         (float)offset);
+    };
+    if (hidden <= 2048) launch.template operator()<1>();
+    else if (hidden <= 4096) launch.template operator()<2>();
+    else launch.template operator()<4>();
+    return;
+  }
   hy_dispatch(x, "sandwich_norm_res32", [&]<typename T>() {
     hipLaunchKernelGGL(sandwich_norm_res32_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
                        reinterpret_cast<T*>(x.data_ptr()), residual.data_ptr<float>(),
@@ -304,14 +318,12 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
   TORCH_CHECK(tau > 0);
   const auto dt = q.scalar_type();
   TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt && z.scalar_type() == dt);
-  const size_t lds = sizeof(float) * ((size_t)3 * kGlaTB * D + (size_t)kGlaTB * 64);
-  const dim3 grid((DV + 63) / 64, H, B);
+  const dim3 grid((DV + 15) / 16, H, B);
   const float q_scale = 1.0f / sqrtf((float)D);
   hy_dispatch(q, "gla_recurrence", [&]<typename T>() {
     auto launch = [&]<int DPL>() {
-      auto kern = gla_recurrence_kernel<T, DPL>;
-      allow_lds(kern, lds);
-      hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), o.data_ptr<float>(),
+      hipLaunchKernelGGL((gla_recurrence_kernel<T, DPL>), grid, dim3(256), 0, hy_stream(),
+                         o.data_ptr<float>(),
                          reinterpret_cast<const T*>(q.data_ptr()), q.stride(0),
                          reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
                          reinterpret_cast<const T*>(v.data_ptr()), v.stride(0),
@@ -320,10 +332,10 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
                          slots.data_ptr<int>(), fresh.data_ptr<int>(), H, D, DV,
                          (float)(1.0 / tau), q_scale);
     };
-    if (D <= 32) launch.template operator()<8>();
-    else if (D <= 64) launch.template operator()<16>();
-    else if (D <= 128) launch.template operator()<32>();
-    else launch.template operator()<64>();
+    if (D <= 32) launch.template operator()<2>();
+    else if (D <= 64) launch.template operator()<4>();
+    else if (D <= 128) launch.template operator()<8>();
+    else launch.template operator()<16>();
   });
 }
 

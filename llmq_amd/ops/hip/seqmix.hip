@@ -64,6 +64,70 @@ __global__ void sandwich_norm_res32_kernel(T* __restrict__ x, float* __restrict_
     xr[i] = from_f32<T>(rr[i] * inv2 * (to_f32(w_pre[i]) + offset));
 }
 
+// The same sandwich for bf16 rows of up to CH * 2048 elements, a multiple of
+// 8 wide: every thread keeps its 8-element granules of the updated residual
+// in registers, so x, the residual and the two weights cross memory exactly
+// once, in 16-byte accesses.
+template <int CH>
+__global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
+    __hip_bfloat16* __restrict__ x, float* __restrict__ residual,
+    const __hip_bfloat16* __restrict__ w_post, const __hip_bfloat16* __restrict__ w_pre,
+    int hidden, float eps, float offset) {
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  __hip_bfloat16* xr = x + row * hidden;
+  float* rr = residual + row * hidden;
+  float xv[CH][8], rv[CH][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const Vec8<__hip_bfloat16> v = load16(xr + i);
+      const float4 ra = *reinterpret_cast<const float4*>(rr + i);
+      const float4 rb = *reinterpret_cast<const float4*>(rr + i + 4);
+      rv[c][0] = ra.x; rv[c][1] = ra.y; rv[c][2] = ra.z; rv[c][3] = ra.w;
+      rv[c][4] = rb.x; rv[c][5] = rb.y; rv[c][6] = rb.z; rv[c][7] = rb.w;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        xv[c][j] = to_f32(v.data[j]);
+        ss += xv[c][j] * xv[c][j];
+      }
+    }
+  }
+  ss = block_reduce_sum(ss, red);
+  const float inv1 = 1.0f / sqrtf(ss / hidden + eps);
+  float ss2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const Vec8<__hip_bfloat16> wv = load16(w_post + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        rv[c][j] += xv[c][j] * inv1 * (to_f32(wv.data[j]) + offset);
+        ss2 += rv[c][j] * rv[c][j];
+      }
+      *reinterpret_cast<float4*>(rr + i) = make_float4(rv[c][0], rv[c][1], rv[c][2], rv[c][3]);
+      *reinterpret_cast<float4*>(rr + i + 4) = make_float4(rv[c][4], rv[c][5], rv[c][6], rv[c][7]);
+    }
+  }
+  ss2 = block_reduce_sum(ss2, red);
+  const float inv2 = 1.0f / sqrtf(ss2 / hidden + eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const Vec8<__hip_bfloat16> wv = load16(w_pre + i);
+      Vec8<__hip_bfloat16> ov;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        ov.data[j] = __float2bfloat16(rv[c][j] * inv2 * (to_f32(wv.data[j]) + offset));
+      store16(xr + i, ov);
+    }
+  }
+}
+
 // ------------------------------------------------------------ activations --
 // Scalar fallback of act_and_mul for widths that are not a multiple of the
 // 16-byte vector (the vector kernel lives in elementwise.hip).
@@ -617,13 +681,17 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
 // with a_t = sigmoid(z_t + z_bias)^(1/tau) per key channel, state S in fp32
 // [D, DV] living in a per-sequence slot between steps.
 //
-// Value columns evolve independently, so the grid splits DV: a wave owns 16
-// columns, its lanes are 16 columns x 4 key groups (key channel d = kg + 4 i
-// sits in register S[i]); o is a 4-lane shuffle reduce. The workgroup's 4
-// waves share 16-token stages of q, k, decay (computed once, fp32) and v in
-// LDS. Sequential over tokens, parallel over (sequence, head, 64 columns).
-// A sequence whose portion starts at position 0 (fresh != 0) starts from a
-// zero state without reading its slot, so reused slots need no clearing.
+// Value columns evolve independently, so the grid splits DV: a workgroup owns
+// 16 columns of one (sequence, head). Its 256 threads are 16 columns x 16 key
+// groups (4 per wave); a thread keeps DPL consecutive key channels of one
+// column in registers, so a token costs it DPL multiply-adds per product.
+// The partial o of a wave (4-lane shuffle reduce) goes to LDS and the four
+// waves' partials are summed once per 16-token stage. Each stage's q, k and
+// decay (computed once, fp32: exp(log_sigmoid(z) / tau)) and v sit in LDS,
+// zero-padded to 16*DPL channels. Sequential over tokens, parallel over
+// (sequence, head, 16 columns). A sequence whose portion starts at position 0
+// (fresh != 0) starts from a zero state without reading its slot, so reused
+// slots need no clearing.
 constexpr int kGlaTB = 16;
 
 template <typename T, int DPL>
@@ -639,16 +707,17 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
     const int* __restrict__ slots,          // [B]
     const int* __restrict__ fresh,          // [B]
     int H, int D, int DV, float inv_tau, float q_scale) {
-  extern __shared__ float smem[];
-  float* qs = smem;                 // [TB][D]
-  float* ks = qs + kGlaTB * D;      // [TB][D]
-  float* as = ks + kGlaTB * D;      // [TB][D]
-  float* vs = as + kGlaTB * D;      // [TB][64]
+  constexpr int DP = 16 * DPL;          // padded key channels
+  __shared__ __align__(16) float qs[kGlaTB * DP];
+  __shared__ __align__(16) float ks[kGlaTB * DP];
+  __shared__ __align__(16) float as[kGlaTB * DP];
+  __shared__ float vs[kGlaTB * 16];
+  __shared__ float po[kGlaTB * 4 * 16];
   const int b = blockIdx.z, h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int col = (lane & 15) + 16 * w;      // column within the 64-wide tile
-  const int c = blockIdx.x * 64 + col;
-  const int kg = lane >> 4;
+  const int colw = lane & 15, kg = lane >> 4;
+  const int c = blockIdx.x * 16 + colw;
+  const int d0 = (w * 4 + kg) * DPL;
   const int row0 = cu[b];
   const int n = cu[b + 1] - row0;
   const long sbase = ((long)slots[b] * H + h) * D * (long)DV;
@@ -656,54 +725,77 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
   const bool use_old = fresh[b] == 0;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
-    const int d = kg + 4 * i;
+    const int d = d0 + i;
     S[i] = (use_old && d < D && c < DV) ? state[sbase + (long)d * DV + c] : 0.f;
   }
   for (int t0 = 0; t0 < n; t0 += kGlaTB) {
     const int nt = min(kGlaTB, n - t0);
     __syncthreads();
-    for (int idx = tid; idx < nt * D; idx += 256) {
-      const int tt = idx / D, d = idx % D;
-      const long row = row0 + t0 + tt;
-      qs[idx] = to_f32(q[row * q_stride + (long)h * D + d]) * q_scale;
-      ks[idx] = to_f32(k[row * k_stride + (long)h * D + d]);
-      const float zz = to_f32(z[row * z_stride + (long)h * D + d]) + z_bias[h * D + d];
-      // log sigmoid(zz) = -(max(-zz, 0) + log1p(exp(-|zz|)))
-      const float ls = -(fmaxf(-zz, 0.f) + log1pf(expf(-fabsf(zz))));
-      as[idx] = expf(ls * inv_tau);
+    for (int idx = tid; idx < nt * DP; idx += 256) {
+      const int tt = idx / DP, d = idx % DP;
+      float qv = 0.f, kv = 0.f, av = 0.f;
+      if (d < D) {
+        const long row = row0 + t0 + tt;
+        qv = to_f32(q[row * q_stride + (long)h * D + d]) * q_scale;
+        kv = to_f32(k[row * k_stride + (long)h * D + d]);
+        const float zz = to_f32(z[row * z_stride + (long)h * D + d]) + z_bias[h * D + d];
+        // log sigmoid(zz) = -(max(-zz, 0) + log1p(exp(-|zz|)))
+        const float ls = -(fmaxf(-zz, 0.f) + log1pf(expf(-fabsf(zz))));
+        av = expf(ls * inv_tau);
+      }
+      qs[idx] = qv;
+      ks[idx] = kv;
+      as[idx] = av;
     }
-    for (int idx = tid; idx < nt * 64; idx += 256) {
-      const int tt = idx >> 6, cc = idx & 63;
-      const int gc = blockIdx.x * 64 + cc;
-      vs[idx] = gc < DV
-          ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc])
-          : 0.f;
+    if (tid < nt * 16) {
+      const int tt = tid >> 4, cc = tid & 15;
+      const int gc = blockIdx.x * 16 + cc;
+      vs[tid] = gc < DV ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc]) : 0.f;
     }
     __syncthreads();
     for (int tt = 0; tt < nt; ++tt) {
-      const float vv = vs[tt * 64 + col];
-      const float* qa = qs + tt * D;
-      const float* ka = ks + tt * D;
-      const float* aa = as + tt * D;
+      const float vv = vs[tt * 16 + colw];
+      const float* qa = qs + tt * DP + d0;
+      const float* ka = ks + tt * DP + d0;
+      const float* aa = as + tt * DP + d0;
       float part = 0.f;
+      if constexpr (DPL % 4 == 0) {
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) {
-        const int d = kg + 4 * i;
-        if (d < D) {
-          S[i] = aa[d] * S[i] + ka[d] * vv;
-          part += S[i] * qa[d];
+        for (int i = 0; i < DPL; i += 4) {
+          const float4 a4 = *reinterpret_cast<const float4*>(aa + i);
+          const float4 k4 = *reinterpret_cast<const float4*>(ka + i);
+          const float4 q4 = *reinterpret_cast<const float4*>(qa + i);
+          S[i] = a4.x * S[i] + k4.x * vv;
+          S[i + 1] = a4.y * S[i + 1] + k4.y * vv;
+          S[i + 2] = a4.z * S[i + 2] + k4.z * vv;
+          S[i + 3] = a4.w * S[i + 3] + k4.w * vv;
+          part += S[i] * q4.x + S[i + 1] * q4.y + S[i + 2] * q4.z + S[i + 3] * q4.w;
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < DPL; ++i) {
+          S[i] = aa[i] * S[i] + ka[i] * vv;
+          part += S[i] * qa[i];
         }
       }
       part += __shfl_xor(part, 16, WAVE);
       part += __shfl_xor(part, 32, WAVE);
-      if (kg == 0 && c < DV)
-        o[((long)(row0 + t0 + tt) * H + h) * DV + c] = part;
+      if (kg == 0) po[(tt * 4 + w) * 16 + colw] = part;
+    }
+    __syncthreads();
+    if (tid < nt * 16) {
+      const int tt = tid >> 4, cc = tid & 15;
+      const int gc = blockIdx.x * 16 + cc;
+      if (gc < DV) {
+        const float* pp = po + tt * 64 + cc;
+        o[((long)(row0 + t0 + tt) * H + h) * DV + gc] = (pp[0] + pp[16]) + (pp[32] + pp[48]);
+      }
     }
   }
   if (c < DV) {
 #pragma unroll
     for (int i = 0; i < DPL; ++i) {
-      const int d = kg + 4 * i;
+      const int d = d0 + i;
       if (d < D) state[sbase + (long)d * DV + c] = S[i];
     }
   }
