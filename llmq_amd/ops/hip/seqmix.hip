@@ -687,7 +687,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
 // column in registers, so a token costs it DPL multiply-adds per product.
 // The partial o of a wave (4-lane shuffle reduce) goes to LDS and the four
 // waves' partials are summed once per 16-token stage. Each stage's q, k and
-// decay (computed once, fp32: exp(log_sigmoid(z) / tau)) and v sit in LDS,
+// decay (computed once per stage, fp32: exp(log_sigmoid(z) / tau)) and v sit in LDS,
 // zero-padded to 16*DPL channels. Sequential over tokens, parallel over
 // (sequence, head, 16 columns). A sequence whose portion starts at position 0
 // (fresh != 0) starts from a zero state without reading its slot, so reused
@@ -728,31 +728,61 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
     const int d = d0 + i;
     S[i] = (use_old && d < D && c < DV) ? state[sbase + (long)d * DV + c] : 0.f;
   }
+  // A thread stages exactly DPL (token, channel) pairs per 16-token stage
+  // (idx = tid + 256 j). The next stage's raw q, k, z and v are fetched into
+  // registers before the current stage's token loop and turned into LDS
+  // contents (scale, decay) after it: memory latency hides behind the math.
+  float rq[DPL], rk[DPL], rz[DPL], rv = 0.f;
+  auto fetch = [&](int t0) {
+    const int nt = min(kGlaTB, n - t0);
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) {
+      const int idx = tid + 256 * j;
+      const int tt = idx / DP, d = idx % DP;
+      rq[j] = rk[j] = rz[j] = 0.f;
+      if (tt < nt && d < D) {
+        const long row = row0 + t0 + tt;
+        rq[j] = to_f32(q[row * q_stride + (long)h * D + d]);
+        rk[j] = to_f32(k[row * k_stride + (long)h * D + d]);
+        rz[j] = to_f32(z[row * z_stride + (long)h * D + d]);
+      }
+    }
+    rv = 0.f;
+    if (tid < nt * 16) {
+      const int gc = blockIdx.x * 16 + (tid & 15);
+      if (gc < DV) rv = to_f32(v[(long)(row0 + t0 + (tid >> 4)) * v_stride + (long)h * DV + gc]);
+    }
+  };
+  if (n > 0) fetch(0);
   for (int t0 = 0; t0 < n; t0 += kGlaTB) {
     const int nt = min(kGlaTB, n - t0);
     __syncthreads();
-    for (int idx = tid; idx < nt * DP; idx += 256) {
-      const int tt = idx / DP, d = idx % DP;
-      float qv = 0.f, kv = 0.f, av = 0.f;
+#pragma unroll
+    for (int j = 0; j < DPL; ++j) {
+      const int idx = tid + 256 * j;
+      const int d = idx % DP;
+      float av = 0.f;
       if (d < D) {
-        const long row = row0 + t0 + tt;
-        qv = to_f32(q[row * q_stride + (long)h * D + d]) * q_scale;
-        kv = to_f32(k[row * k_stride + (long)h * D + d]);
-        const float zz = to_f32(z[row * z_stride + (long)h * D + d]) + z_bias[h * D + d];
-        // log sigmoid(zz) = -(max(-zz, 0) + log1p(exp(-|zz|)))
-        const float ls = -(fmaxf(-zz, 0.f) + log1pf(expf(-fabsf(zz))));
-        av = expf(ls * inv_tau);
+        const float zz = rz[j] + z_bias[h * D + d];
+        // log sigmoid(zz) = min(zz, 0) - log1p(exp(-|zz|)); fp32 models take
+        // the accurate library functions, bf16 models the hardware exp/log
+        // (a few ulp of fp32, far below the rounding of their inputs)
+        if constexpr (std::is_same_v<T, float>) {
+          const float ls = fminf(zz, 0.f) - log1pf(expf(-fabsf(zz)));
+          av = expf(ls * inv_tau);
+        } else {
+          const float ls = fminf(zz, 0.f) - __logf(1.0f + __expf(-fabsf(zz)));
+          av = __expf(ls * inv_tau);
+        }
       }
-      qs[idx] = qv;
-      ks[idx] = kv;
+      qs[idx] = rq[j] * q_scale;
+      ks[idx] = rk[j];
       as[idx] = av;
     }
-    if (tid < nt * 16) {
-      const int tt = tid >> 4, cc = tid & 15;
-      const int gc = blockIdx.x * 16 + cc;
-      vs[tid] = gc < DV ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc]) : 0.f;
-    }
+    vs[tid] = rv;
     __syncthreads();
+    if (t0 + kGlaTB < n) fetch(t0 + kGlaTB);
+#pragma unroll 4
     for (int tt = 0; tt < nt; ++tt) {
       const float vv = vs[tt * 16 + colw];
       const float* qa = qs + tt * DP + d0;
