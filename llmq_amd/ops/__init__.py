@@ -30,6 +30,15 @@ def _try_load_extension() -> None:
     if _EXT_TRIED:
         return
     _EXT_TRIED = True
+    # A build in this very process (ops.build.build / ensure) has already
+    # loaded the library it produced: loading the copied file again would
+    # register the namespace twice, which aborts the process.
+    try:
+        torch.ops.llmq_amd.rmsnorm  # noqa: B018
+        _EXT = torch.ops.llmq_amd
+        return
+    except (AttributeError, RuntimeError):
+        pass
     here = Path(__file__).parent
     override = os.environ.get("LLMQ_OPS_SO")
     if override:
@@ -349,6 +358,12 @@ def _try_load_hybrid() -> None:
     if _HY_TRIED:
         return
     _HY_TRIED = True
+    try:  # built (and thereby loaded) earlier in this process
+        torch.ops.llmq_amd_hybrid.rmsnorm_cast  # noqa: B018
+        _HY = torch.ops.llmq_amd_hybrid
+        return
+    except (AttributeError, RuntimeError):
+        pass
     here = Path(__file__).parent
     override = os.environ.get("LLMQ_HYBRID_OPS_SO")
     candidates = [Path(override)] if override else sorted(here.glob("_hip_hybrid*.so"))
