@@ -220,6 +220,25 @@ def clear(queue_name, include_results, yes) -> None:
     monitor.clear_queue(queue_name, include_results, yes)
 
 
+# ----------------------------------------------------------------- trace --
+
+
+@cli.command("trace-run")
+@click.option("--model", required=True, help="Checkpoint folder (config.json + model.safetensors)")
+@click.option("--dtype", type=click.Choice(["bfloat16", "float32"]), default="bfloat16")
+@click.option("--out", required=True, help="Folder the <step>.f32 logits files are written to")
+@click.option("--max-tokens", type=int, required=True,
+              help="Most tokens live requests hold at any time (sizes the KV pool)")
+def trace_run(model, dtype, out, max_tokens) -> None:
+    """Replay a token trace (JSON steps on stdin) through the engine and
+    write the logits of the wanted positions — teacher-forced, nothing is
+    sampled. Same program as bin/trace_run."""
+    from llmq_amd.engine.trace_replay import main as replay_main
+
+    raise SystemExit(replay_main(
+        ["--model", model, "--dtype", dtype, "--out", out, "--max-tokens", str(max_tokens)]))
+
+
 # ---------------------------------------------------------------- worker --
 
 
