@@ -527,3 +527,118 @@ def test_trace_runner_cli(tmp_path, mixed_model):
     assert not (tmp_path / "o" / "1.f32").exists()
     got = torch.from_numpy(np.concatenate([a, b]))
     assert_close(got, want[[0, 19, 29]], ("cpu", "float32"))
+
+
+# ------------------------------ kernel envelopes: sizes beyond the models --
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("H,G,D,DV,span", [
+    (4, 2, 32, 16, 24),       # one MFMA k-step, one channel tile
+    (6, 3, 40, 72, 50),       # q/k size not a multiple of 32, five channel tiles
+    (2, 1, 64, 48, 130),
+    (2, 2, 128, 136, 300),    # the widest instantiation
+    (1, 1, 256, 256, 70),
+    (3, 3, 20, 10, 9),        # not a multiple of 8: the fp32-ALU kernel in bf16 too
+])
+def test_attention_ops_against_dense(target, H, G, D, DV, span):
+    """qknorm_vmix_cache + both attention kernels on shuffled pages against
+    dense float64 attention, for portions that start mid-span and mid-page."""
+    from llmq_amd import ops
+
+    device, dtype = target[0], getattr(torch, target[1])
+    g = torch.Generator().manual_seed(H * 1000 + D)
+    bs, L = 16, 333
+    nq, nk, nv = H * D, G * D, G * DV
+    proj = torch.randn(L, nq + nk + nv + H, generator=g).to(dtype)
+    v_first = torch.randn(L, nv, generator=g).to(dtype)
+    qw = (1 + 0.2 * torch.randn(nq, generator=g)).to(dtype)
+    kw = (1 + 0.2 * torch.randn(nk, generator=g)).to(dtype)
+    bias = torch.randn(H, span, generator=g)
+    lam, scale, eps = 0.35, 0.7 / math.sqrt(D), 1e-5
+    nblk = (L + bs - 1) // bs
+    table = (torch.randperm(nblk + 3, generator=g)[:nblk]).to(torch.int32).view(1, -1)
+    kc = torch.zeros(nblk + 3, G, bs, D, dtype=dtype, device=device)
+    vc = torch.zeros(nblk + 3, G, bs, DV, dtype=dtype, device=device)
+    # dense reference
+    pd = proj.double()
+    qn = oracle.plain_rmsnorm(pd[:, :nq], qw.double(), eps).view(L, H, D)
+    kn = oracle.plain_rmsnorm(pd[:, nq:nq + nk], kw.double(), eps).view(L, G, D)
+    vm = ((1 - lam) * pd[:, nq + nk:nq + nk + nv] + lam * v_first.double()).view(L, G, DV)
+    if dtype == torch.bfloat16:   # what the cache holds
+        qn, kn, vm = (t.to(dtype).double() for t in (qn, kn, vm))
+    kh, vh = kn.repeat_interleave(H // G, 1), vm.repeat_interleave(H // G, 1)
+    i = torch.arange(L).view(-1, 1)
+    j = torch.arange(L).view(1, -1)
+    sc = torch.einsum("ihd,jhd->hij", qn, kh) * scale + bias.double()[:, (i - j).clamp(0, span - 1)]
+    sc = sc.masked_fill(~oracle.block_causal_mask(L, span).unsqueeze(0), float("-inf"))
+    want = torch.einsum("hij,jhd->ihd", torch.softmax(sc, -1), vh)
+    want = want * torch.sigmoid(pd[:, nq + nk + nv:]).unsqueeze(-1)
+    # engine ops: portions, the last rows one by one
+    cuts = [0, 5, min(5 + span + 3, 150), 200, 290, 291, 293] + list(range(294, L + 1))
+    got = []
+    for lo, hi in zip(cuts[:-1], cuts[1:]):
+        p = proj[lo:hi].clone().to(device)
+        q, k, v = p[:, :nq], p[:, nq:nq + nk], p[:, nq + nk:nq + nk + nv]
+        gate = p[:, nq + nk + nv:]
+        slots = torch.tensor([int(table[0, t // bs]) * bs + t % bs for t in range(lo, hi)],
+                             dtype=torch.long, device=device)
+        ops.qknorm_vmix_cache(q, k, v, qw.to(device), kw.to(device), v_first[lo:hi].to(device),
+                              lam, kc, vc, slots, eps)
+        q3 = q.view(hi - lo, H, D)
+        if hi - lo == 1 and lo > 0:
+            got.append(ops.chunk_bias_attn_decode(
+                q3, gate, kc, vc, bias.to(device), table.to(device),
+                torch.tensor([hi], dtype=torch.int32, device=device), span, scale))
+        else:
+            got.append(ops.chunk_bias_attn_prefill(
+                q3, gate, kc, vc, bias.to(device), table.to(device),
+                torch.tensor([0, hi - lo], dtype=torch.int32, device=device),
+                torch.tensor([lo], dtype=torch.int32, device=device), hi - lo, span, scale))
+    got = torch.cat(got).double().cpu()
+    err = (got - want).abs().max() / want.abs().max()
+    assert float(err) < (2e-2 if dtype == torch.bfloat16 else 2e-5), float(err)
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("H,D,DV,tau", [(2, 16, 32, 16.0), (3, 40, 72, 4.0), (1, 128, 200, 1.0),
+                                        (1, 256, 24, 0.5), (5, 6, 5, 2.0)])
+def test_gla_ops_against_recurrence(target, H, D, DV, tau):
+    """gla_recurrence + gla_out_norm_gate for several packed sequences with
+    old and fresh slots against the token-by-token float64 recurrence."""
+    from llmq_amd import ops
+
+    device, dtype = target[0], getattr(torch, target[1])
+    g = torch.Generator().manual_seed(D * 7 + DV)
+    lens, slots, fresh = [70, 21, 2, 1], [3, 0, 5, 1], [1, 0, 0, 1]
+    T = sum(lens)
+    q = torch.randn(T, H, D, generator=g).to(dtype)
+    k = torch.randn(T, H, D, generator=g).to(dtype)
+    v = torch.randn(T, H, DV, generator=g).to(dtype)
+    z = (2 * torch.randn(T, H, D, generator=g)).to(dtype)
+    zb = torch.randn(H * D, generator=g)
+    state0 = torch.randn(6, H, D, DV, generator=g)
+    w = (1 + 0.2 * torch.randn(DV, generator=g)).to(dtype)
+    gate = torch.randn(T, H * DV, generator=g).to(dtype)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    st = state0.clone().to(device)
+    o = ops.gla_recurrence(q.to(device), k.to(device), v.to(device), z.to(device), zb.to(device),
+                           st, cu.to(device), torch.tensor(slots, dtype=torch.int32, device=device),
+                           torch.tensor(fresh, dtype=torch.int32, device=device), tau)
+    y = ops.gla_out_norm_gate(o, w.to(device), gate.to(device), 1e-5, dtype)
+    alpha = torch.sigmoid(z.double() + zb.double().view(1, H, D)).pow(1.0 / tau)
+    want_o = torch.empty(T, H, DV, dtype=torch.float64)
+    want_state = state0.double().clone()
+    at = 0
+    for n, slot, fr in zip(lens, slots, fresh):
+        S = torch.zeros(H, D, DV, dtype=torch.float64) if fr else state0[slot].double().clone()
+        for t in range(at, at + n):
+            S = alpha[t].unsqueeze(-1) * S + k[t].double().unsqueeze(-1) * v[t].double().unsqueeze(-2)
+            want_o[t] = torch.einsum("hdv,hd->hv", S, q[t].double() * D ** -0.5)
+        want_state[slot] = S
+        at += n
+    assert float((o.double().cpu() - want_o).abs().max() / want_o.abs().max()) < 1e-5
+    assert float((st.double().cpu() - want_state).abs().max() / want_state.abs().max()) < 1e-5
+    want_y = oracle.plain_rmsnorm(want_o, w.double(), 1e-5).reshape(T, H * DV) * \
+        torch.nn.functional.silu(gate.double())
+    err = float((y.double().cpu() - want_y).abs().max() / want_y.abs().max())
+    assert err < (1e-2 if dtype == torch.bfloat16 else 1e-5), err
