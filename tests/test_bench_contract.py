@@ -87,3 +87,18 @@ def test_bench_tp_mode_two_ranks_gloo():
     # ONE engine's tokens (not 2×): global_batch equals per-engine batch
     assert data["config"]["global_batch"] == 4  # CPU tiny shape
     assert data["value"] > 0
+
+
+@pytest.mark.timeout(300)
+def test_bench_compare_hybrid_option():
+    """--compare-hybrid prints one JSON line per model with prefill and decode
+    throughput and leaves the default workload alone."""
+    proc = subprocess.run(
+        [sys.executable, "bench.py", "--compare-hybrid", "--steps", "3", "--warmup", "1"],
+        capture_output=True, text=True, cwd=REPO, timeout=280,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [l["family"] for l in lines] == ["kakovik", "llama"]
+    for l in lines:
+        assert l["prefill_tokens_per_sec"] > 0 and l["decode_tokens_per_sec"] > 0
