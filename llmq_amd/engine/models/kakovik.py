@@ -153,7 +153,9 @@ class KakovikLM:
             if m.kind != "attention":
                 continue
             rel = lw.t["rel"].float().cpu()
-            rows = [distance_bucket(n, m.bias_rows, m.bias_far) for n in range(m.span)]
+            # distances inside one span, and never beyond the longest context
+            n_dist = min(m.span, self.spec.max_position_embeddings)
+            rows = [distance_bucket(n, m.bias_rows, m.bias_far) for n in range(n_dist)]
             lw.bias = rel[torch.tensor(rows, dtype=torch.long)].t().contiguous().to(self.device)
             lw.lam = float(lw.t["vmix"].float().item())
             if m.v_mix:

@@ -179,8 +179,8 @@ AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optio
   TORCH_CHECK(a.H % a.G == 0, "heads must be a multiple of kv heads");
   TORCH_CHECK(a.DV <= 256, "value size above 256 is not supported");
   TORCH_CHECK(span >= 1 && bias.scalar_type() == at::kFloat && bias.is_contiguous() &&
-              bias.dim() == 2 && bias.size(0) == a.H && bias.size(1) == span,
-              "bias must be fp32 [H, span]");
+              bias.dim() == 2 && bias.size(0) == a.H && bias.size(1) >= 1 && bias.size(1) <= span,
+              "bias must be fp32 [H, n], n = min(span, longest context the engine admits)");
   TORCH_CHECK(q.scalar_type() == out.scalar_type() && q.scalar_type() == k_cache.scalar_type() &&
               q.scalar_type() == v_cache.scalar_type());
   HY_I32(block_tables);
@@ -233,6 +233,7 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const bf*>(k_cache.data_ptr()),
                          reinterpret_cast<const bf*>(v_cache.data_ptr()), bias.data_ptr<float>(),
+                         (int)bias.size(1),
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
                          (int)span, (float)scale);
@@ -256,6 +257,7 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const T*>(k_cache.data_ptr()),
                          reinterpret_cast<const T*>(v_cache.data_ptr()), bias.data_ptr<float>(),
+                         (int)bias.size(1),
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
                          (int)span, (float)scale);
@@ -284,6 +286,7 @@ void chunk_bias_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const T*>(k_cache.data_ptr()),
                          reinterpret_cast<const T*>(v_cache.data_ptr()), bias.data_ptr<float>(),
+                         (int)bias.size(1),
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          context_lens.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs, (int)span,
                          (float)scale);
@@ -318,7 +321,7 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
   TORCH_CHECK(tau > 0);
   const auto dt = q.scalar_type();
   TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt && z.scalar_type() == dt);
-  const dim3 grid((DV + 15) / 16, H, B);
+  const dim3 grid((DV + kGlaCols - 1) / kGlaCols, H, B);
   const float q_scale = 1.0f / sqrtf((float)D);
   hy_dispatch(q, "gla_recurrence", [&]<typename T>() {
     auto launch = [&]<int DPL>() {

@@ -229,7 +229,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     const T* __restrict__ q, long q_stride,
     const T* __restrict__ gate, long g_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const float* __restrict__ bias,        // [H, span]
+    const float* __restrict__ bias, int bias_len,   // [H, bias_len], bias_len = min(span, longest context)
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q,          // [B+1]
     const int* __restrict__ q_start,       // [B] position of a sequence's first query
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const int i = pos0 + w * 4 + r;
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
                        key / span == i / span;
-      const float sc = vis ? s[r] + bias[(long)h * span + (i - key)] : -INFINITY;
+      const float sc = vis ? s[r] + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : -INFINITY;
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -379,7 +379,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const __hip_bfloat16* __restrict__ q, long q_stride,
     const __hip_bfloat16* __restrict__ gate, long g_stride,
     const __hip_bfloat16* __restrict__ k_cache, const __hip_bfloat16* __restrict__ v_cache,
-    const float* __restrict__ bias,        // [H, span]
+    const float* __restrict__ bias, int bias_len,   // [H, bias_len]
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale) {
@@ -432,7 +432,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   const int wave_lo = (wave_first / span) * span;
   const bool wave_rows = w * 16 < rows;
   const int* bt = block_tables + (long)b * bt_stride;
-  const float* bias_h = bias + (long)h * span;
+  const float* bias_h = bias + (long)h * bias_len;
   short* Pw = Ps + w * 2 * 16 * kMfmaKP;
   const bool v_vec = (DV % 8) == 0;
 
@@ -489,7 +489,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     if (tid < 127) {
       // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)
       const int d = pos0 - kt - 63 + tid;
-      Bs[tid] = (d >= 0 && d < span) ? bias_h[d] : 0.f;
+      Bs[tid] = (d >= 0 && d < bias_len) ? bias_h[d] : 0.f;
     }
     __syncthreads();
     if (kt + kMfmaKT <= pos_last) fetch(kt + kMfmaKT);
@@ -600,7 +600,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     const T* __restrict__ q, long q_stride,
     const T* __restrict__ gate, long g_stride,
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
-    const float* __restrict__ bias,
+    const float* __restrict__ bias, int bias_len,
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ context_lens,
     int H, int G, int D, int DV, int block_size, int span, float scale) {
@@ -631,7 +631,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
       const T* kr = k_cache + base * D;
       float s = 0.f;
       for (int d = 0; d < D; ++d) s += Qs[d] * to_f32(kr[d]);
-      sc = s + bias[(long)h * span + (i - key)];
+      sc = s + bias[(long)h * bias_len + min(i - key, bias_len - 1)];
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));  // nk >= 1: finite
     const float corr = expf(m - m_new);
@@ -682,17 +682,18 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
 // [D, DV] living in a per-sequence slot between steps.
 //
 // Value columns evolve independently, so the grid splits DV: a workgroup owns
-// 16 columns of one (sequence, head). Its 256 threads are 16 columns x 16 key
-// groups (4 per wave); a thread keeps DPL consecutive key channels of one
-// column in registers, so a token costs it DPL multiply-adds per product.
-// The partial o of a wave (4-lane shuffle reduce) goes to LDS and the four
+// 32 columns of one (sequence, head), two per thread. Its 256 threads are 16 column pairs x 16 key
+// groups (4 per wave, one lane quad per column); a thread keeps DPL
+// consecutive key channels of one column in registers, so a token costs it
+// DPL multiply-adds per product. The partial o of a wave (quad reduce) goes to LDS and the four
 // waves' partials are summed once per 16-token stage. Each stage's q, k and
 // decay (computed once per stage, fp32: exp(log_sigmoid(z) / tau)) and v sit in LDS,
 // zero-padded to 16*DPL channels. Sequential over tokens, parallel over
-// (sequence, head, 16 columns). A sequence whose portion starts at position 0
+// (sequence, head, 32 columns). A sequence whose portion starts at position 0
 // (fresh != 0) starts from a zero state without reading its slot, so reused
 // slots need no clearing.
 constexpr int kGlaTB = 16;
+constexpr int kGlaCols = 32;   // value columns per workgroup (2 per thread)
 
 template <typename T, int DPL>
 __global__ __launch_bounds__(256) void gla_recurrence_kernel(
@@ -711,28 +712,31 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
   __shared__ __align__(16) float qs[kGlaTB * DP];
   __shared__ __align__(16) float ks[kGlaTB * DP];
   __shared__ __align__(16) float as[kGlaTB * DP];
-  __shared__ float vs[kGlaTB * 16];
-  __shared__ float po[kGlaTB * 4 * 16];
+  __shared__ float vs[kGlaTB * kGlaCols];
+  __shared__ float po[kGlaTB * 4 * kGlaCols];
   const int b = blockIdx.z, h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int colw = lane & 15, kg = lane >> 4;
-  const int c = blockIdx.x * 16 + colw;
+  // a column's 4 key groups sit in one lane quad: their reduce is two DPP
+  // quad permutes, no LDS traffic
+  const int colw = lane >> 2, kg = lane & 3;
+  const int c0 = blockIdx.x * kGlaCols + colw, c1 = c0 + 16;
   const int d0 = (w * 4 + kg) * DPL;
   const int row0 = cu[b];
   const int n = cu[b + 1] - row0;
   const long sbase = ((long)slots[b] * H + h) * D * (long)DV;
-  float S[DPL];
+  float S0[DPL], S1[DPL];
   const bool use_old = fresh[b] == 0;
 #pragma unroll
   for (int i = 0; i < DPL; ++i) {
     const int d = d0 + i;
-    S[i] = (use_old && d < D && c < DV) ? state[sbase + (long)d * DV + c] : 0.f;
+    S0[i] = (use_old && d < D && c0 < DV) ? state[sbase + (long)d * DV + c0] : 0.f;
+    S1[i] = (use_old && d < D && c1 < DV) ? state[sbase + (long)d * DV + c1] : 0.f;
   }
   // A thread stages exactly DPL (token, channel) pairs per 16-token stage
-  // (idx = tid + 256 j). The next stage's raw q, k, z and v are fetched into
-  // registers before the current stage's token loop and turned into LDS
-  // contents (scale, decay) after it: memory latency hides behind the math.
-  float rq[DPL], rk[DPL], rz[DPL], rv = 0.f;
+  // (idx = tid + 256 j) and two values. The next stage's raw q, k, z and v
+  // are fetched into registers before the current stage's token loop and
+  // turned into LDS contents (scale, decay) after it.
+  float rq[DPL], rk[DPL], rz[DPL], rv[2];
   auto fetch = [&](int t0) {
     const int nt = min(kGlaTB, n - t0);
 #pragma unroll
@@ -747,10 +751,12 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
         rz[j] = to_f32(z[row * z_stride + (long)h * D + d]);
       }
     }
-    rv = 0.f;
-    if (tid < nt * 16) {
-      const int gc = blockIdx.x * 16 + (tid & 15);
-      if (gc < DV) rv = to_f32(v[(long)(row0 + t0 + (tid >> 4)) * v_stride + (long)h * DV + gc]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int idx = tid + 256 * j;
+      const int tt = idx / kGlaCols, gc = blockIdx.x * kGlaCols + idx % kGlaCols;
+      rv[j] = (tt < nt && gc < DV)
+          ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc]) : 0.f;
     }
   };
   if (n > 0) fetch(0);
@@ -779,55 +785,71 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
       ks[idx] = rk[j];
       as[idx] = av;
     }
-    vs[tid] = rv;
+    vs[tid] = rv[0];
+    vs[tid + 256] = rv[1];
     __syncthreads();
     if (t0 + kGlaTB < n) fetch(t0 + kGlaTB);
 #pragma unroll 4
     for (int tt = 0; tt < nt; ++tt) {
-      const float vv = vs[tt * 16 + colw];
+      const float v0 = vs[tt * kGlaCols + colw];
+      const float v1 = vs[tt * kGlaCols + 16 + colw];
       const float* qa = qs + tt * DP + d0;
       const float* ka = ks + tt * DP + d0;
       const float* aa = as + tt * DP + d0;
-      float part = 0.f;
+      float p0 = 0.f, p1 = 0.f;
       if constexpr (DPL % 4 == 0) {
 #pragma unroll
         for (int i = 0; i < DPL; i += 4) {
           const float4 a4 = *reinterpret_cast<const float4*>(aa + i);
           const float4 k4 = *reinterpret_cast<const float4*>(ka + i);
           const float4 q4 = *reinterpret_cast<const float4*>(qa + i);
-          S[i] = a4.x * S[i] + k4.x * vv;
-          S[i + 1] = a4.y * S[i + 1] + k4.y * vv;
-          S[i + 2] = a4.z * S[i + 2] + k4.z * vv;
-          S[i + 3] = a4.w * S[i + 3] + k4.w * vv;
-          part += S[i] * q4.x + S[i + 1] * q4.y + S[i + 2] * q4.z + S[i + 3] * q4.w;
+          S0[i] = a4.x * S0[i] + k4.x * v0;
+          S0[i + 1] = a4.y * S0[i + 1] + k4.y * v0;
+          S0[i + 2] = a4.z * S0[i + 2] + k4.z * v0;
+          S0[i + 3] = a4.w * S0[i + 3] + k4.w * v0;
+          p0 += S0[i] * q4.x + S0[i + 1] * q4.y + S0[i + 2] * q4.z + S0[i + 3] * q4.w;
+          S1[i] = a4.x * S1[i] + k4.x * v1;
+          S1[i + 1] = a4.y * S1[i + 1] + k4.y * v1;
+          S1[i + 2] = a4.z * S1[i + 2] + k4.z * v1;
+          S1[i + 3] = a4.w * S1[i + 3] + k4.w * v1;
+          p1 += S1[i] * q4.x + S1[i + 1] * q4.y + S1[i + 2] * q4.z + S1[i + 3] * q4.w;
         }
       } else {
 #pragma unroll
         for (int i = 0; i < DPL; ++i) {
-          S[i] = aa[i] * S[i] + ka[i] * vv;
-          part += S[i] * qa[i];
+          S0[i] = aa[i] * S0[i] + ka[i] * v0;
+          p0 += S0[i] * qa[i];
+          S1[i] = aa[i] * S1[i] + ka[i] * v1;
+          p1 += S1[i] * qa[i];
         }
       }
-      part += __shfl_xor(part, 16, WAVE);
-      part += __shfl_xor(part, 32, WAVE);
-      if (kg == 0) po[(tt * 4 + w) * 16 + colw] = part;
+      p0 += __shfl_xor(p0, 1, WAVE);
+      p0 += __shfl_xor(p0, 2, WAVE);
+      p1 += __shfl_xor(p1, 1, WAVE);
+      p1 += __shfl_xor(p1, 2, WAVE);
+      if (kg == 0) {
+        po[(tt * 4 + w) * kGlaCols + colw] = p0;
+        po[(tt * 4 + w) * kGlaCols + 16 + colw] = p1;
+      }
     }
     __syncthreads();
-    if (tid < nt * 16) {
-      const int tt = tid >> 4, cc = tid & 15;
-      const int gc = blockIdx.x * 16 + cc;
-      if (gc < DV) {
-        const float* pp = po + tt * 64 + cc;
-        o[((long)(row0 + t0 + tt) * H + h) * DV + gc] = (pp[0] + pp[16]) + (pp[32] + pp[48]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int idx = tid + 256 * j;
+      const int tt = idx / kGlaCols, cc = idx % kGlaCols;
+      const int gc = blockIdx.x * kGlaCols + cc;
+      if (tt < nt && gc < DV) {
+        const float* pp = po + tt * 4 * kGlaCols + cc;
+        o[((long)(row0 + t0 + tt) * H + h) * DV + gc] =
+            (pp[0] + pp[kGlaCols]) + (pp[2 * kGlaCols] + pp[3 * kGlaCols]);
       }
     }
   }
-  if (c < DV) {
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) {
-      const int d = d0 + i;
-      if (d < D) state[sbase + (long)d * DV + c] = S[i];
-    }
+  for (int i = 0; i < DPL; ++i) {
+    const int d = d0 + i;
+    if (d < D && c0 < DV) state[sbase + (long)d * DV + c0] = S0[i];
+    if (d < D && c1 < DV) state[sbase + (long)d * DV + c1] = S1[i];
   }
 }
 
