@@ -23,8 +23,10 @@ logger = logging.getLogger(__name__)
 class KVCache:
     """Uniform models pass (num_layers, num_kv_heads, head_dim); models whose
     layers differ pass ``layout``: one (kv_heads, k_dim, v_dim) per layer, or
-    None for a layer that caches no keys (its k/v entries are None). All
-    layers share block ids, so one block table serves every layer."""
+    None for a layer that caches no keys (its k/v entries are None); v_dim 0
+    means the layer's values are read out of its key rows (latent caches), so
+    only k is allocated. All layers share block ids, so one block table
+    serves every layer."""
 
     def __init__(
         self,
@@ -59,6 +61,7 @@ class KVCache:
             )
             self.v.append(
                 torch.zeros(num_blocks, heads, block_size, v_dim, device=device, dtype=dtype)
+                if v_dim else None
             )
 
     @staticmethod

@@ -380,10 +380,243 @@ HYBRID_PRESETS = {
 }
 
 
+# ---------------------------------------------------------------------------
+# Kosalorn: a looped hybrid decoder. One norm per layer feeds a sequence
+# mixer (latent attention or an HGRN2 recurrence) and a feed-forward (dense
+# or a mixture of experts) in parallel, each behind a sigmoid gate, followed
+# by a per-layer token-indexed side input. A range of layers may run several
+# times in a row with the same weights (each pass with its own cache/state).
+
+
+@dataclass
+class RotarySpec:
+    """Rotary positions on the first `dims` coordinates of a vector: pair i
+    turns by position * base^(-2i/dims). layout "half": pair (i, i+dims/2);
+    "interleaved": pair (2i, 2i+1)."""
+
+    base: float
+    dims: int
+    layout: str = "half"
+
+
+@dataclass
+class LatentAttnSpec:
+    """Attention over a shared low-rank latent: per token only the normed
+    latent (kv_rank) and one rotated key part (rot_dim) are cached; per-head
+    keys and values are linear maps of the latent. q_rank > 0: the query goes
+    through a normed latent too. window 0 = causal, else position i sees
+    j with 0 <= i - j < window."""
+
+    heads: int
+    dim: int            # per-head unrotated q/k size
+    rot_dim: int        # per-head rotated q size = shared rotated key size
+    vdim: int
+    kv_rank: int
+    scale: float
+    rot: RotarySpec = None
+    q_rank: int = 0
+    window: int = 0
+    kind: str = "latent_attention"
+
+
+@dataclass
+class HGRN2Spec:
+    """Linear attention whose forget gate f = l + (1-l)*sigmoid(.) also sets
+    the write strength: S <- diag(f) S + (1-f) v^T, o = S^T q."""
+
+    heads: int
+    dim: int
+    vdim: int
+    kind: str = "hgrn2"
+
+
+@dataclass
+class MoESpec:
+    """Mixture of gated feed-forward experts: sigmoid router scores, the
+    `top` best experts per token, the score scales the expert's INPUT."""
+
+    experts: int
+    top: int
+    ff: int             # per-expert inner size
+
+
+@dataclass
+class KosalornLayerSpec:
+    mixer: object                 # LatentAttnSpec | HGRN2Spec
+    ff: int = 0                   # dense feed-forward inner size (0 = none)
+    moe: Optional[MoESpec] = None
+
+
+@dataclass
+class KosalornSpec:
+    name: str
+    family: str                   # "kosalorn"
+    vocab_size: int
+    hidden_size: int
+    layers: list = field(default_factory=list)
+    rms_eps: float = 1e-6
+    side_dim: int = 0             # per-layer token side input width (0 = none)
+    loop_start: int = 0           # layers [loop_start, loop_stop) run
+    loop_stop: int = 0            # loop_times times in a row
+    loop_times: int = 1
+    max_position_embeddings: int = 1 << 17
+    tied_embeddings: bool = False
+    eos_token_id: int = 2
+    bos_token_id: int = 1
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def runs(self) -> list:
+        """Execution order: [(layer index, adds the embedding output first)].
+        A looped layer appears once per pass; every entry owns its own cache
+        or state."""
+        n = len(self.layers)
+        a, b, times = self.loop_start, self.loop_stop, self.loop_times
+        if times <= 1 or b <= a:
+            return [(i, False) for i in range(n)]
+        order = [(i, False) for i in range(a)]
+        for p in range(times):
+            order += [(i, p > 0 and i == a) for i in range(a, b)]
+        return order + [(i, False) for i in range(b, n)]
+
+    def param_count(self) -> int:
+        w = self.hidden_size
+        total = 2 * self.vocab_size * w + 2
+        total += self.vocab_size * self.side_dim * len(self.layers)
+        for ls in self.layers:
+            m = ls.mixer
+            total += 1 + 2 * (w * w + w)
+            if m.kind == "hgrn2":
+                nk, nv = m.heads * m.dim, m.heads * m.vdim
+                total += 2 * nk * w + 2 * nk + nv * w + m.vdim + w * nv
+            else:
+                nq = m.heads * (m.dim + m.rot_dim)
+                total += (m.q_rank * (w + 1 + nq)) if m.q_rank else nq * w
+                total += (m.kv_rank + m.rot_dim) * w + m.kv_rank
+                total += m.kv_rank * m.heads * (m.dim + m.vdim) + w * m.heads * m.vdim
+            if ls.ff:
+                total += 3 * w * ls.ff
+            if ls.moe:
+                total += ls.moe.experts * (3 * w * ls.moe.ff + w)
+            if self.side_dim:
+                total += 2 * w * self.side_dim + w
+        return total
+
+
+def kosalorn_spec_from_config(cfg: dict, name: str) -> KosalornSpec:
+    """Kosalorn config.json -> KosalornSpec. Every size and constant comes
+    from the config; the layer type fixes the rotary layout and whether the
+    query has a latent."""
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc, kind = lc["mixer"], lc["type"]
+        if kind in ("latent_attention", "latent_attention_2"):
+            rot = mc["rot"]
+            mask = mc.get("mask")
+            mixer = LatentAttnSpec(
+                heads=int(mc["heads"]), dim=int(mc["dim"]), rot_dim=int(mc["rot_dim"]),
+                vdim=int(mc["vdim"]), kv_rank=int(mc["kv_rank"]), scale=float(mc["scale"]),
+                rot=RotarySpec(base=float(rot["base"]), dims=int(rot["dims"]),
+                               layout="half" if kind == "latent_attention" else "interleaved"),
+                q_rank=int(mc.get("q_rank", 0)) if kind == "latent_attention" else 0,
+                window=int(mask["size"]) if mask else 0,
+            )
+            if kind == "latent_attention" and not mixer.q_rank:
+                raise ValueError(f"layer {i}: latent_attention needs q_rank")
+            if mixer.rot.dims > mixer.rot_dim or mixer.rot.dims % 2:
+                raise ValueError(f"layer {i}: rot.dims must be even and at most rot_dim")
+        elif kind == "hgrn2":
+            mixer = HGRN2Spec(heads=int(mc["heads"]), dim=int(mc["dim"]), vdim=int(mc["vdim"]))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp = lc.get("mlp")
+        ff, moe = 0, None
+        if mlp is not None:
+            if mlp.get("kind", "dense") == "dense":
+                ff = int(mlp["ff"])
+            elif mlp["kind"] == "moe":
+                moe = MoESpec(experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]),
+                              ff=int(mlp["expert"]["ff"]))
+                if not 1 <= moe.top <= moe.experts:
+                    raise ValueError(f"layer {i}: top must be within 1..experts")
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp['kind']!r}")
+        layers.append(KosalornLayerSpec(mixer=mixer, ff=ff, moe=moe))
+    loop = cfg.get("loop") or {}
+    side = cfg.get("token_side") or {}
+    spec = KosalornSpec(
+        name=name, family="kosalorn", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers, rms_eps=float(cfg["norm"]["eps"]),
+        side_dim=int(side.get("dim", 0)),
+        loop_start=int(loop.get("start", 0)), loop_stop=int(loop.get("stop", 0)),
+        loop_times=int(loop.get("times", 1)),
+    )
+    if not 0 <= spec.loop_start <= spec.loop_stop <= len(layers):
+        raise ValueError("loop range outside the layer list")
+    return spec
+
+
+def _kosalorn(name, vocab, width, n_layers, heads, dim, rot_dim, vdim, kv_rank, q_rank, ff,
+              window=0, rec_every=4, rec_heads=None, rec_dim=None, rec_vdim=None,
+              moe_every=0, experts=8, top=2, expert_ff=None, side_dim=0, loop=None, **kw):
+    """Preset builder: every `rec_every`-th layer is an HGRN2 layer, the
+    others latent attention (alternating the windowed query-latent form and
+    the causal direct-query form); every `moe_every`-th feed-forward is a
+    mixture of experts, the others dense."""
+    layers = []
+    for i in range(n_layers):
+        if rec_every and i % rec_every == rec_every - 1:
+            mixer = HGRN2Spec(heads=rec_heads or heads, dim=rec_dim or dim, vdim=rec_vdim or vdim)
+        elif i % 2 == 0:
+            mixer = LatentAttnSpec(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim,
+                                   kv_rank=kv_rank, scale=(dim + rot_dim) ** -0.5,
+                                   rot=RotarySpec(250000.0, rot_dim, "half"),
+                                   q_rank=q_rank, window=window)
+        else:
+            mixer = LatentAttnSpec(heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim,
+                                   kv_rank=kv_rank, scale=(dim + rot_dim) ** -0.5,
+                                   rot=RotarySpec(500000.0, rot_dim, "interleaved"))
+        if moe_every and i % moe_every == moe_every - 1:
+            layers.append(KosalornLayerSpec(mixer, moe=MoESpec(experts, top, expert_ff or ff)))
+        else:
+            layers.append(KosalornLayerSpec(mixer, ff=ff))
+    a, b, times = loop or (0, 0, 1)
+    return KosalornSpec(name=name, family="kosalorn", vocab_size=vocab, hidden_size=width,
+                        layers=layers, side_dim=side_dim, loop_start=a, loop_stop=b,
+                        loop_times=times, **kw)
+
+
+KOSALORN_PRESETS = {
+    # CPU/GPU test config: every mixer and feed-forward kind, a looped range
+    "tiny-kosalorn": _kosalorn("tiny-kosalorn", 512, 64, 4, 4, 16, 8, 24, 40, 24, 96,
+                               window=24, rec_every=3, rec_heads=2, rec_dim=16, rec_vdim=32,
+                               moe_every=2, experts=6, top=2, expert_ff=32, side_dim=8,
+                               loop=(1, 3, 2)),
+    # benchmark configs at the layer sizes of llama-3.2-1b / -3b (the closest
+    # existing models): same width, head count, feed-forward and depth; the
+    # head size is split into an unrotated and a rotated part, the latent is
+    # four heads wide
+    "kosalorn-1b": _kosalorn("kosalorn-1b", 128256, 2048, 16, 32, 32, 32, 64, 192, 768, 8192,
+                             window=2048, rec_every=4, rec_heads=16, rec_dim=64, rec_vdim=128),
+    "kosalorn-3b": _kosalorn("kosalorn-3b", 128256, 3072, 28, 24, 64, 64, 128, 192, 1536, 8192,
+                             window=2048, rec_every=4, rec_heads=12, rec_dim=128, rec_vdim=256),
+    # the same with every second feed-forward a mixture of 8 experts, 2 per
+    # token, each a quarter of the dense inner size
+    "kosalorn-1b-moe": _kosalorn("kosalorn-1b-moe", 128256, 2048, 16, 32, 32, 32, 64, 192, 768,
+                                 8192, window=2048, rec_every=4, rec_heads=16, rec_dim=64,
+                                 rec_vdim=128, moe_every=2, experts=8, top=2, expert_ff=2048,
+                                 side_dim=64),
+}
+
+
 def spec_from_hf_config(path: Path, name: str) -> ModelSpec:
     """Build a spec from a HF checkpoint directory's config.json."""
     with open(path / "config.json", "r", encoding="utf-8") as fh:
         cfg = json.load(fh)
+    if str(cfg.get("architecture", "")).lower() == "kosalorn":
+        return kosalorn_spec_from_config(cfg, name)
     if str(cfg.get("architecture", "")).lower() == "kakovik":
         st = path / "model.safetensors"
         return kakovik_spec_from_config(
@@ -461,7 +694,9 @@ def resolve_spec(model: str) -> ModelSpec:
         return PRESETS[key]
     if key in HYBRID_PRESETS:
         return HYBRID_PRESETS[key]
+    if key in KOSALORN_PRESETS:
+        return KOSALORN_PRESETS[key]
     raise ValueError(
         f"Unknown model '{model}'. Provide a checkpoint directory with config.json "
-        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(ALIASES)}"
+        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(KOSALORN_PRESETS) + sorted(ALIASES)}"
     )

@@ -1,6 +1,7 @@
 """Model registry: spec family → model class."""
 
 from llmq_amd.engine.models.kakovik import KakovikLM
+from llmq_amd.engine.models.kosalorn import KosalornLM
 from llmq_amd.engine.models.llama import CausalLM
 
 MODEL_CLASSES = {
@@ -9,6 +10,7 @@ MODEL_CLASSES = {
     "gemma2": CausalLM,
     "mistral": CausalLM,
     "kakovik": KakovikLM,
+    "kosalorn": KosalornLM,
 }
 
 
@@ -19,4 +21,4 @@ def model_class_for(spec):
         raise ValueError(f"no model class registered for family {spec.family!r}") from None
 
 
-__all__ = ["CausalLM", "KakovikLM", "MODEL_CLASSES", "model_class_for"]
+__all__ = ["CausalLM", "KakovikLM", "KosalornLM", "MODEL_CLASSES", "model_class_for"]

@@ -160,4 +160,103 @@ def load_kakovik_weights(model, path: Path) -> None:
     logger.info("loaded %d tensors from %s", len(tensors), path)
 
 
-_FAMILY_LOADERS = {"kakovik": load_kakovik_weights}
+def _read_all(path: Path) -> Dict[str, torch.Tensor]:
+    from safetensors import safe_open  # noqa: PLC0415
+
+    files = sorted(path.glob("*.safetensors"))
+    if not files:
+        raise FileNotFoundError(f"no .safetensors under {path}")
+    tensors: Dict[str, torch.Tensor] = {}
+    for f in files:
+        with safe_open(str(f), framework="pt", device="cpu") as sf:
+            for name in sf.keys():
+                tensors[name] = sf.get_tensor(name)
+    return tensors
+
+
+def load_kosalorn_weights(model, path: Path) -> None:
+    """Kosalorn checkpoint names -> the packed in-tree tensors.
+
+    Checkpoint: 'embed', 'embed.norm', 'head', 'final.norm', 'side.embed', and
+    per layer 'l<i>.norm1', the gates 'l<i>.rg1' / '.rg1.b' / '.rg2' /
+    '.rg2.b', the mixer under 'l<i>.mix.', the feed-forward under
+    'l<i>.mlp.' (experts 'e<j>.'), the side input under 'l<i>.side.'; linear
+    weights are [out, in]. Packing: mixer input projections ‖ rg1 ‖ rg2 ->
+    'in' (segments at multiples of 8 rows), feed-forward gate‖up -> gate_up,
+    experts stacked [E, ...]; uk / uv split per head."""
+    tensors = _read_all(path)
+    used = set()
+
+    def get(name: str) -> torch.Tensor:
+        if name not in tensors:
+            raise KeyError(f"missing tensor {name}")
+        used.add(name)
+        return tensors[name]
+
+    def copy_(dst: torch.Tensor, src: torch.Tensor) -> None:
+        if dst.shape != src.shape:
+            raise ValueError(f"shape mismatch: {tuple(dst.shape)} vs {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    spec = model.spec
+    copy_(model.embedding, get("embed"))
+    copy_(model.embed_norm, get("embed.norm"))
+    copy_(model.lm_head, get("head"))
+    copy_(model.final_norm, get("final.norm"))
+    if spec.side_dim:
+        copy_(model.side_embed, get("side.embed"))
+    for i, (ls, lw) in enumerate(zip(spec.layers, model.layers)):
+        p, t, m = f"l{i}.", lw.t, ls.mixer
+        mx = p + "mix."
+        copy_(t["norm1"], get(p + "norm1"))
+
+        def put(seg: str, src: torch.Tensor, lw=lw, t=t) -> None:
+            at, n = lw.seg[seg]
+            copy_(t["in"][at:at + n], src)
+
+        t["in"].zero_()  # alignment rows between segments
+        if m.kind == "hgrn2":
+            put("q", get(mx + "q"))
+            put("f", get(mx + "f"))
+            put("v", get(mx + "v"))
+            copy_(t["f_b"], get(mx + "f.b"))
+            copy_(t["lower"], get(mx + "lower"))
+            copy_(t["norm"], get(mx + "norm"))
+        else:
+            if m.q_rank:
+                put("dq", get(mx + "dq"))
+                copy_(t["dq_norm"], get(mx + "dq.norm"))
+                copy_(t["uq"], get(mx + "uq"))
+            else:
+                put("q", get(mx + "q"))
+            put("dkv", get(mx + "dkv"))
+            copy_(t["dkv_norm"], get(mx + "dkv.norm"))
+            copy_(t["uk"], get(mx + "uk").view(m.heads, m.dim, m.kv_rank))
+            copy_(t["uv"], get(mx + "uv").view(m.heads, m.vdim, m.kv_rank))
+        copy_(t["o"], get(mx + "o"))
+        put("rg1", get(p + "rg1"))
+        copy_(t["rg1_b"], get(p + "rg1.b"))
+        if ls.ff or ls.moe:
+            put("rg2", get(p + "rg2"))
+            copy_(t["rg2_b"], get(p + "rg2.b"))
+        if ls.ff:
+            copy_(t["gate_up"], torch.cat([get(p + "mlp.gate"), get(p + "mlp.up")], dim=0))
+            copy_(t["down"], get(p + "mlp.down"))
+        if ls.moe:
+            copy_(t["router"], get(p + "mlp.router"))
+            for e in range(ls.moe.experts):
+                ep = f"{p}mlp.e{e}."
+                copy_(t["e_gate_up"][e], torch.cat([get(ep + "gate"), get(ep + "up")], dim=0))
+                copy_(t["e_down"][e], get(ep + "down"))
+        if spec.side_dim:
+            copy_(t["side_gate"], get(p + "side.gate"))
+            copy_(t["side_proj"], get(p + "side.proj"))
+            copy_(t["side_norm"], get(p + "side.norm"))
+    unused = sorted(set(tensors) - used)
+    if unused:
+        raise ValueError(f"checkpoint tensors the model does not know: {unused[:8]}")
+    model.finalize()
+    logger.info("loaded %d tensors from %s", len(tensors), path)
+
+
+_FAMILY_LOADERS = {"kakovik": load_kakovik_weights, "kosalorn": load_kosalorn_weights}

@@ -442,14 +442,20 @@ def qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, lam: float, k_cache, v_cache,
                                 slot_mapping, eps)
 
 
+# mask modes of the paged attention kernels: keys of the query's own span of
+# positions (counted from 0), or the `span` newest positions up to the query
+_MASK_BLOCK, _MASK_WINDOW = 0, 1
+_NO_WINDOW = (1 << 31) - 1
+
+
 def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q, q_start,
                             max_q: int, span: int, scale: float) -> torch.Tensor:
     """Block-local causal attention + per-distance bias for packed prompt
     portions; keys/values come from the paged cache. q [T, H, D] → [T, H, DV]."""
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
-        _HY.chunk_bias_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
-                                    q_start, int(max_q), int(span), float(scale))
+        _HY.paged_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
+                               q_start, int(max_q), int(span), float(scale), _MASK_BLOCK)
         return out
     return torch_ref.chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables,
                                              cu_q, q_start, span, scale)
@@ -460,8 +466,8 @@ def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, contex
     """The single-token form: query b sits at position context_lens[b]-1."""
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
-        _HY.chunk_bias_attn_decode(out, q, gate, k_cache, v_cache, bias, block_tables,
-                                   context_lens, int(span), float(scale))
+        _HY.paged_attn_decode(out, q, gate, k_cache, v_cache, bias, block_tables,
+                              context_lens, int(span), float(scale), _MASK_BLOCK)
         return out
     return torch_ref.chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables,
                                             context_lens, span, scale)
@@ -470,11 +476,24 @@ def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, contex
 def gla_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau: float) -> torch.Tensor:
     """Gated-linear-attention recurrence over packed sequences; returns o
     [T, H, DV] fp32 and advances state [slots, H, D, DV] in place."""
+    return gated_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau=tau,
+                            q_scale=1.0 / (q.shape[2] ** 0.5))
+
+
+def gated_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau: float = 1.0,
+                     lower=None, q_silu: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+    """Diagonal-decay recurrence S <- diag(a) S + w v^T, o = S^T (q_scale * act(q))
+    over packed sequences, state [slots, H, D, DV] fp32 advanced in place.
+    lower None (gated linear attention): a = sigmoid(z + b)^(1/tau), w = k.
+    lower [H*D] fp32 (HGRN2): a = l + (1 - l) * sigmoid(z + b), w = 1 - a and
+    k is not read. q_silu applies SiLU to q first. Returns o [T, H, DV] fp32."""
     if _use_hybrid(q):
         o = torch.empty(q.shape[0], q.shape[1], v.shape[2], dtype=torch.float32, device=q.device)
-        _HY.gla_recurrence(o, q, k, v, z, z_bias, state, cu, slots, fresh, float(tau))
+        _HY.gla_recurrence(o, q, k, v, z, z_bias, state, cu, slots, fresh, float(tau),
+                           lower, bool(q_silu), float(q_scale))
         return o
-    return torch_ref.gla_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau)
+    return torch_ref.gated_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau, lower,
+                                      q_silu, q_scale)
 
 
 def gla_out_norm_gate(o, weight, gate, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
@@ -485,3 +504,129 @@ def gla_out_norm_gate(o, weight, gate, eps: float, out_dtype: torch.dtype) -> to
         _HY.gla_out_norm_gate(out, o, weight, gate, eps)
         return out
     return torch_ref.gla_out_norm_gate(o, weight, gate, eps, out_dtype)
+
+
+def head_norm(o, weight, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-head RMSNorm of a recurrence output o [T, H, DV] fp32 x weight [DV]."""
+    if _use_hybrid(o):
+        T, H, DV = o.shape
+        out = torch.empty(T, H * DV, dtype=out_dtype, device=o.device)
+        _HY.gla_out_norm_gate(out, o, weight, None, eps)
+        return out
+    return torch_ref.head_norm(o, weight, eps, out_dtype)
+
+
+def window_attn_prefill(q, k_cache, v_cache, dv: int, block_tables, cu_q, q_start, max_q: int,
+                        window: int, scale: float) -> torch.Tensor:
+    """Softmax attention of packed prompt portions over the paged cache:
+    query at position i sees keys j <= i with i - j < window (window 0:
+    every j <= i). v_cache None: the first dv channels of a key row are its
+    value (latent caches). q [T, H, D] -> [T, H, dv]."""
+    if _use_hybrid(q):
+        out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
+        _HY.paged_attn_prefill(out, q, None, k_cache, v_cache, None, block_tables, cu_q, q_start,
+                               int(max_q), int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW)
+        return out
+    return torch_ref.window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start,
+                                         window, scale)
+
+
+def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens, window: int,
+                       scale: float) -> torch.Tensor:
+    """The single-token form: query b sits at position context_lens[b]-1."""
+    if _use_hybrid(q):
+        out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
+        _HY.paged_attn_decode(out, q, None, k_cache, v_cache, None, block_tables, context_lens,
+                              int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW)
+        return out
+    return torch_ref.window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens,
+                                        window, scale)
+
+
+def latent_rope_pack(q, q_lat, ckr, c_w, inv_freq, positions, k_cache, slots, dim: int,
+                     rot_dims: int, interleaved: bool, eps: float) -> torch.Tensor:
+    """Latent attention, between the projections and the attention kernel:
+    rotary positions (fp32 angles position * inv_freq[i]) on the rotated part
+    of q [T, H, dim+DR] and of ckr [T, R+DR], RMSNorm of the latent, the
+    packed query q_lat ‖ rotated part [T, H, R+DR] returned, and latent ‖
+    rotated key part scattered into the paged cache [blocks, 1, bs, R+DR]."""
+    if _use_hybrid(q):
+        T, H, _ = q.shape
+        out = torch.empty(T, H, ckr.shape[1], dtype=q.dtype, device=q.device)
+        _HY.latent_rope_pack(out, q, q_lat, ckr, c_w, inv_freq, positions, k_cache, slots,
+                             int(dim), int(rot_dims), bool(interleaved), float(eps))
+        return out
+    return torch_ref.latent_rope_pack(q, q_lat, ckr, c_w, inv_freq, positions, k_cache, slots,
+                                      dim, rot_dims, interleaved, eps)
+
+
+def gated_residual_add(res, y1, g1, b1, y2, g2, b2, out_dtype: torch.dtype) -> torch.Tensor:
+    """res (fp32, in place) += sigmoid(g1 + b1) * y1 [+ sigmoid(g2 + b2) * y2];
+    returns the updated rows rounded to out_dtype. g1/g2 may be column
+    slices of a wider projection output."""
+    if _use_hybrid(res):
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        _HY.gated_residual_add(out, res, y1, g1, b1, y2, g2, b2)
+        return out
+    return torch_ref.gated_residual_add(res, y1, g1, b1, y2, g2, b2, out_dtype)
+
+
+def side_gate_mul(a, table, tokens, offset: int) -> torch.Tensor:
+    """gelu_tanh(a) * table[tokens, offset : offset + a.shape[1]]."""
+    if _use_hybrid(a):
+        out = torch.empty_like(a)
+        _HY.side_gate_mul(out, a, table, tokens, int(offset))
+        return out
+    return torch_ref.side_gate_mul(a, table, tokens, offset)
+
+
+def sigmoid_topk(logits, top: int):
+    """Router scores sigmoid(logits) in fp32 and their `top` largest per
+    row: (indices int32 [T, top], scores fp32 [T, top])."""
+    if _use_hybrid(logits):
+        T = logits.shape[0]
+        idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+        _HY.sigmoid_topk(idx, w, logits, int(top))
+        return idx, w
+    return torch_ref.sigmoid_topk(logits, top)
+
+
+# rows (token, expert) pairs up to which the expert mixture runs as
+# per-row matrix-vector kernels (no host sync, graph-capturable)
+MOE_GEMV_MAX_ROWS = 64
+
+
+def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False) -> torch.Tensor:
+    """Sum over a token's chosen experts of down_e(silu(gate_e x) * up_e x)
+    with x = w * h (the router score scales the expert's INPUT).
+    h [T, W]; idx/w [T, top]; gate_up [E, 2F, W]; down [E, W, F].
+
+    Few rows (or sync_free, for captured decode graphs): one matrix-vector
+    kernel pair that reads each row's expert weights. Many rows: rows
+    sorted by expert and one GEMM pair per expert on contiguous slices (the
+    per-expert row counts cross to the host once)."""
+    T, top = idx.shape
+    if h.is_cuda and (sync_free or T * top <= MOE_GEMV_MAX_ROWS):
+        _use_hybrid(h)
+        F_ = down.shape[2]
+        hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
+        _HY.moe_gate_up_gemv(hmid, h, idx, w, gate_up)
+        y = torch.empty_like(h)
+        _HY.moe_down_gemv(y, hmid, idx, down)
+        return y
+    E = gate_up.shape[0]
+    flat = idx.reshape(-1).long()
+    order = torch.sort(flat, stable=True).indices
+    counts = torch.bincount(flat, minlength=E).tolist()
+    xs = (h.float()[order // top] * w.reshape(-1)[order].unsqueeze(1)).to(h.dtype)
+    ys = torch.empty_like(xs)
+    at = 0
+    for e, n in enumerate(counts):
+        if n:
+            act = act_and_mul(torch.nn.functional.linear(xs[at:at + n], gate_up[e]))
+            ys[at:at + n] = torch.nn.functional.linear(act, down[e])
+            at += n
+    inv = torch.empty_like(order)
+    inv[order] = torch.arange(order.numel(), device=order.device)
+    return ys[inv].view(T, top, -1).float().sum(dim=1).to(h.dtype)

@@ -34,23 +34,27 @@ void allow_lds(K kernel, size_t bytes) {
 
 void rmsnorm_cast(at::Tensor out, at::Tensor in, at::Tensor weight, double eps, double offset) {
   HY_GPU(in);
-  TORCH_CHECK(in.is_contiguous() && out.is_contiguous() && weight.is_contiguous());
+  // in: contiguous, or 2-D rows with a stride (a column slice of a wider matrix)
+  TORCH_CHECK(out.is_contiguous() && weight.is_contiguous());
+  TORCH_CHECK(in.is_contiguous() || (in.dim() == 2 && in.stride(1) == 1),
+              "rmsnorm_cast: in must be contiguous or row-strided 2-D");
   const int hidden = in.size(-1);
   TORCH_CHECK(out.sizes() == in.sizes() && weight.numel() == hidden);
   TORCH_CHECK(weight.scalar_type() == out.scalar_type(), "weight dtype must equal out dtype");
   const long rows = in.numel() / hidden;
   if (rows == 0) return;
+  const long in_stride = in.is_contiguous() ? hidden : in.stride(0);
   hy_dispatch(out, "rmsnorm_cast", [&]<typename TO>() {
     if (in.scalar_type() == at::kFloat) {
       hipLaunchKernelGGL((rmsnorm_cast_kernel<float, TO>), dim3(rows), dim3(256), 0, hy_stream(),
-                         reinterpret_cast<TO*>(out.data_ptr()), in.data_ptr<float>(),
+                         reinterpret_cast<TO*>(out.data_ptr()), in.data_ptr<float>(), in_stride,
                          reinterpret_cast<const TO*>(weight.data_ptr()), hidden, (float)eps,
                          (float)offset);
     } else {
       TORCH_CHECK(in.scalar_type() == out.scalar_type(), "rmsnorm_cast: in must be fp32 or out's dtype");
       hipLaunchKernelGGL((rmsnorm_cast_kernel<TO, TO>), dim3(rows), dim3(256), 0, hy_stream(),
                          reinterpret_cast<TO*>(out.data_ptr()),
-                         reinterpret_cast<const TO*>(in.data_ptr()),
+                         reinterpret_cast<const TO*>(in.data_ptr()), in_stride,
                          reinterpret_cast<const TO*>(weight.data_ptr()), hidden, (float)eps,
                          (float)offset);
     }
@@ -162,27 +166,46 @@ void qknorm_vmix_cache(at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor q_w,
   });
 }
 
-struct AttnDims { int H, G, D, DV, bs; };
+// v_row: value row stride in elements (DV for a value cache of its own, D
+// when values are the first DV channels of the key rows); vptr: where they sit
+struct AttnDims { int H, G, D, DV, bs, v_row; const void* vptr; const float* bias; int bias_len; };
 
 AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optional<at::Tensor>& gate,
-                    const at::Tensor& k_cache, const at::Tensor& v_cache, const at::Tensor& bias,
-                    const at::Tensor& block_tables, long span) {
+                    const at::Tensor& k_cache, const std::optional<at::Tensor>& v_cache,
+                    const std::optional<at::Tensor>& bias, const at::Tensor& block_tables,
+                    long span, long mask_mode) {
   HY_GPU(q);
   TORCH_CHECK(q.dim() == 3 && out.dim() == 3, "q [T, H, D], out [T, H, DV]");
   HY_INNER(q); HY_INNER(out);
-  AttnDims a{(int)q.size(1), (int)k_cache.size(1), (int)q.size(2), (int)v_cache.size(3),
-             (int)k_cache.size(2)};
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous());
+  AttnDims a{(int)q.size(1), (int)k_cache.size(1), (int)q.size(2), (int)out.size(2),
+             (int)k_cache.size(2), 0, nullptr, nullptr, 1};
+  TORCH_CHECK(mask_mode == kMaskBlock || mask_mode == kMaskWindow, "unknown mask mode");
   TORCH_CHECK(q.stride(1) == a.D && out.stride(1) == a.DV, "heads must be packed");
-  TORCH_CHECK(k_cache.is_contiguous() && v_cache.is_contiguous());
-  TORCH_CHECK(k_cache.size(3) == a.D && v_cache.size(1) == a.G && v_cache.size(2) == a.bs);
-  TORCH_CHECK(out.size(0) == q.size(0) && out.size(1) == a.H && out.size(2) == a.DV);
+  TORCH_CHECK(k_cache.size(3) == a.D, "query and key sizes differ");
+  if (v_cache.has_value()) {
+    TORCH_CHECK(v_cache->dim() == 4 && v_cache->is_contiguous() && v_cache->size(0) == k_cache.size(0) &&
+                v_cache->size(1) == a.G && v_cache->size(2) == a.bs && v_cache->size(3) == a.DV &&
+                v_cache->scalar_type() == q.scalar_type(), "value cache does not match");
+    a.v_row = a.DV;
+    a.vptr = v_cache->data_ptr();
+  } else {
+    TORCH_CHECK(a.DV <= a.D, "values read from key rows cannot be wider than the rows");
+    a.v_row = a.D;
+    a.vptr = k_cache.data_ptr();
+  }
+  TORCH_CHECK(out.size(0) == q.size(0) && out.size(1) == a.H);
   TORCH_CHECK(a.H % a.G == 0, "heads must be a multiple of kv heads");
-  TORCH_CHECK(a.DV <= 256, "value size above 256 is not supported");
-  TORCH_CHECK(span >= 1 && bias.scalar_type() == at::kFloat && bias.is_contiguous() &&
-              bias.dim() == 2 && bias.size(0) == a.H && bias.size(1) >= 1 && bias.size(1) <= span,
-              "bias must be fp32 [H, n], n = min(span, longest context the engine admits)");
-  TORCH_CHECK(q.scalar_type() == out.scalar_type() && q.scalar_type() == k_cache.scalar_type() &&
-              q.scalar_type() == v_cache.scalar_type());
+  TORCH_CHECK(a.DV >= 1 && a.DV <= 256, "value size above 256 is not supported");
+  TORCH_CHECK(span >= 1);
+  if (bias.has_value()) {
+    TORCH_CHECK(bias->scalar_type() == at::kFloat && bias->is_contiguous() && bias->dim() == 2 &&
+                bias->size(0) == a.H && bias->size(1) >= 1 && bias->size(1) <= span,
+                "bias must be fp32 [H, n], n = min(span, longest context the engine admits)");
+    a.bias = bias->data_ptr<float>();
+    a.bias_len = (int)bias->size(1);
+  }
+  TORCH_CHECK(q.scalar_type() == out.scalar_type() && q.scalar_type() == k_cache.scalar_type());
   HY_I32(block_tables);
   TORCH_CHECK(block_tables.dim() == 2);
   if (gate.has_value()) {
@@ -199,12 +222,13 @@ void dispatch_nv(int DV, F&& f) {
   else f.template operator()<4>();
 }
 
-void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,
-                             at::Tensor k_cache, at::Tensor v_cache, at::Tensor bias,
-                             at::Tensor block_tables, at::Tensor cu_q, at::Tensor q_start,
-                             int64_t max_q, int64_t span, double scale) {
+void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,
+                        at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
+                        const std::optional<at::Tensor>& bias, at::Tensor block_tables,
+                        at::Tensor cu_q, at::Tensor q_start, int64_t max_q, int64_t span,
+                        double scale, int64_t mask_mode) {
   if (q.size(0) == 0) return;
-  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span);
+  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode);
   HY_I32(cu_q); HY_I32(q_start);
   const int B = q_start.numel();
   TORCH_CHECK(cu_q.numel() == B + 1 && block_tables.size(0) == B && max_q >= 1);
@@ -232,11 +256,10 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
                          gate.has_value() ? reinterpret_cast<const bf*>(gate->data_ptr()) : nullptr,
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const bf*>(k_cache.data_ptr()),
-                         reinterpret_cast<const bf*>(v_cache.data_ptr()), bias.data_ptr<float>(),
-                         (int)bias.size(1),
+                         reinterpret_cast<const bf*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode);
     };
     if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
     else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
@@ -256,21 +279,20 @@ void chunk_bias_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<a
                          gate.has_value() ? reinterpret_cast<const T*>(gate->data_ptr()) : nullptr,
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const T*>(k_cache.data_ptr()),
-                         reinterpret_cast<const T*>(v_cache.data_ptr()), bias.data_ptr<float>(),
-                         (int)bias.size(1),
+                         reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode);
     });
   });
 }
 
-void chunk_bias_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,
-                            at::Tensor k_cache, at::Tensor v_cache, at::Tensor bias,
-                            at::Tensor block_tables, at::Tensor context_lens, int64_t span,
-                            double scale) {
+void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,
+                       at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
+                       const std::optional<at::Tensor>& bias, at::Tensor block_tables,
+                       at::Tensor context_lens, int64_t span, double scale, int64_t mask_mode) {
   if (q.size(0) == 0) return;
-  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span);
+  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode);
   HY_I32(context_lens);
   const int B = q.size(0);
   TORCH_CHECK(context_lens.numel() == B && block_tables.size(0) == B);
@@ -285,23 +307,27 @@ void chunk_bias_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at
                          gate.has_value() ? reinterpret_cast<const T*>(gate->data_ptr()) : nullptr,
                          gate.has_value() ? gate->stride(0) : 0L,
                          reinterpret_cast<const T*>(k_cache.data_ptr()),
-                         reinterpret_cast<const T*>(v_cache.data_ptr()), bias.data_ptr<float>(),
-                         (int)bias.size(1),
+                         reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          context_lens.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs, (int)span,
-                         (float)scale);
+                         (float)scale, a.v_row, (int)mask_mode);
     });
   });
 }
 
 // q, k, z: [T, H, D]; v: [T, H, DV] (row-strided views); o: [T, H, DV] fp32;
 // state: [slots, H, D, DV] fp32.
-void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor z,
-                    at::Tensor z_bias, at::Tensor state, at::Tensor cu, at::Tensor slots,
-                    at::Tensor fresh, double tau) {
+// lower given: the HGRN2 form (no key); q_silu: SiLU on q inside the kernel.
+void gla_recurrence(at::Tensor o, at::Tensor q, const std::optional<at::Tensor>& k_opt,
+                    at::Tensor v, at::Tensor z, at::Tensor z_bias, at::Tensor state, at::Tensor cu,
+                    at::Tensor slots, at::Tensor fresh, double tau,
+                    const std::optional<at::Tensor>& lower, bool q_silu, double q_scale_arg) {
   HY_GPU(q);
   const long T_ = q.size(0);
   if (T_ == 0) return;
+  TORCH_CHECK(k_opt.has_value() != lower.has_value(),
+              "a key (gated linear attention) or a lower bound (HGRN2), not both");
+  const at::Tensor& k = k_opt.has_value() ? *k_opt : q;   // q stands in for shape checks
   TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && v.dim() == 3 && z.dim() == 3 && o.dim() == 3);
   HY_INNER(q); HY_INNER(k); HY_INNER(v); HY_INNER(z);
   const int H = q.size(1), D = q.size(2), DV = v.size(2);
@@ -309,6 +335,12 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
   TORCH_CHECK(v.size(0) == T_ && v.size(1) == H);
   TORCH_CHECK(q.stride(1) == D && k.stride(1) == D && z.stride(1) == D && v.stride(1) == DV,
               "heads must be packed");
+  const float* lower_ptr = nullptr;
+  if (lower.has_value()) {
+    TORCH_CHECK(lower->scalar_type() == at::kFloat && lower->is_contiguous() &&
+                lower->numel() == (long)H * D && lower->is_cuda(), "lower must be fp32 [H*D]");
+    lower_ptr = lower->data_ptr<float>();
+  }
   TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous() && o.size(0) == T_ &&
               o.size(1) == H && o.size(2) == DV);
   TORCH_CHECK(state.scalar_type() == at::kFloat && state.is_contiguous() && state.dim() == 4 &&
@@ -322,18 +354,19 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
   const auto dt = q.scalar_type();
   TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt && z.scalar_type() == dt);
   const dim3 grid((DV + kGlaCols - 1) / kGlaCols, H, B);
-  const float q_scale = 1.0f / sqrtf((float)D);
+  const float q_scale = (float)q_scale_arg;
+  const bool has_k = k_opt.has_value();
   hy_dispatch(q, "gla_recurrence", [&]<typename T>() {
     auto launch = [&]<int DPL>() {
       hipLaunchKernelGGL((gla_recurrence_kernel<T, DPL>), grid, dim3(256), 0, hy_stream(),
                          o.data_ptr<float>(),
                          reinterpret_cast<const T*>(q.data_ptr()), q.stride(0),
-                         reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
+                         has_k ? reinterpret_cast<const T*>(k.data_ptr()) : nullptr, k.stride(0),
                          reinterpret_cast<const T*>(v.data_ptr()), v.stride(0),
                          reinterpret_cast<const T*>(z.data_ptr()), z.stride(0),
                          z_bias.data_ptr<float>(), state.data_ptr<float>(), cu.data_ptr<int>(),
                          slots.data_ptr<int>(), fresh.data_ptr<int>(), H, D, DV,
-                         (float)(1.0 / tau), q_scale);
+                         (float)(1.0 / tau), q_scale, lower_ptr, (int)q_silu);
     };
     if (D <= 32) launch.template operator()<2>();
     else if (D <= 64) launch.template operator()<4>();
@@ -342,22 +375,201 @@ void gla_recurrence(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::
   });
 }
 
-void gla_out_norm_gate(at::Tensor out, at::Tensor o, at::Tensor weight, at::Tensor gate, double eps) {
+void gla_out_norm_gate(at::Tensor out, at::Tensor o, at::Tensor weight,
+                       const std::optional<at::Tensor>& gate_opt, double eps) {
   HY_GPU(o);
   TORCH_CHECK(o.dim() == 3 && o.scalar_type() == at::kFloat && o.is_contiguous());
   const long T_ = o.size(0);
   if (T_ == 0) return;
   const int H = o.size(1), DV = o.size(2);
   TORCH_CHECK(out.dim() == 2 && out.size(0) == T_ && out.size(1) == (long)H * DV && out.stride(1) == 1);
-  TORCH_CHECK(gate.dim() == 2 && gate.size(0) == T_ && gate.size(1) == (long)H * DV && gate.stride(1) == 1);
+  const void* gate_ptr = nullptr;
+  long gate_stride = 0;
+  if (gate_opt.has_value()) {
+    const at::Tensor& gate = *gate_opt;
+    TORCH_CHECK(gate.dim() == 2 && gate.size(0) == T_ && gate.size(1) == (long)H * DV &&
+                gate.stride(1) == 1 && gate.scalar_type() == out.scalar_type());
+    gate_ptr = gate.data_ptr();
+    gate_stride = gate.stride(0);
+  }
   TORCH_CHECK(weight.numel() == DV && weight.is_contiguous());
-  TORCH_CHECK(gate.scalar_type() == out.scalar_type() && weight.scalar_type() == out.scalar_type());
+  TORCH_CHECK(weight.scalar_type() == out.scalar_type());
   hy_dispatch(out, "gla_out_norm_gate", [&]<typename T>() {
     hipLaunchKernelGGL(gla_out_norm_gate_kernel<T>, dim3(T_), dim3(256), 0, hy_stream(),
                        reinterpret_cast<T*>(out.data_ptr()), out.stride(0), o.data_ptr<float>(),
                        reinterpret_cast<const T*>(weight.data_ptr()),
-                       reinterpret_cast<const T*>(gate.data_ptr()), gate.stride(0), H, DV,
-                       (float)eps);
+                       reinterpret_cast<const T*>(gate_ptr), gate_stride, H, DV, (float)eps);
+  });
+}
+
+// ---- latent attention: rotary + latent norm + packed query + cache scatter
+void latent_rope_pack(at::Tensor out, at::Tensor q, at::Tensor q_lat, at::Tensor ckr,
+                      at::Tensor c_w, at::Tensor inv_freq, at::Tensor positions,
+                      at::Tensor k_cache, at::Tensor slots, int64_t dim, int64_t rot_dims,
+                      bool interleaved, double eps) {
+  HY_GPU(q);
+  const long T_ = q.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(q.dim() == 3 && q_lat.dim() == 3 && ckr.dim() == 2 && out.dim() == 3);
+  HY_INNER(q); HY_INNER(q_lat); HY_INNER(ckr);
+  const int H = q.size(1), R = q_lat.size(2);
+  const int DR = (int)q.size(2) - (int)dim;
+  TORCH_CHECK(dim >= 0 && DR >= 1, "q must be [T, H, dim + rot part]");
+  TORCH_CHECK(q_lat.size(0) == T_ && q_lat.size(1) == H && ckr.size(0) == T_ && ckr.size(1) == R + DR);
+  TORCH_CHECK(out.is_contiguous() && out.size(0) == T_ && out.size(1) == H && out.size(2) == R + DR);
+  TORCH_CHECK(rot_dims >= 2 && rot_dims % 2 == 0 && rot_dims <= DR, "rot_dims must be even, at most the rotated part");
+  TORCH_CHECK(inv_freq.scalar_type() == at::kFloat && inv_freq.is_contiguous() &&
+              inv_freq.numel() == rot_dims / 2 && inv_freq.is_cuda());
+  TORCH_CHECK(c_w.numel() == R && c_w.is_contiguous());
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() && positions.numel() == T_);
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.numel() == T_);
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && k_cache.size(1) == 1 &&
+              k_cache.size(3) == R + DR, "latent cache must be [blocks, 1, block, R + rot part]");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(q_lat.scalar_type() == dt && ckr.scalar_type() == dt && c_w.scalar_type() == dt &&
+              out.scalar_type() == dt && k_cache.scalar_type() == dt,
+              "latent_rope_pack: one dtype for activations, weights and cache");
+  hy_dispatch(q, "latent_rope_pack", [&]<typename T>() {
+    hipLaunchKernelGGL(latent_rope_pack_kernel<T>, dim3(T_), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()),
+                       reinterpret_cast<const T*>(q.data_ptr()), q.stride(0), q.stride(1),
+                       reinterpret_cast<const T*>(q_lat.data_ptr()), q_lat.stride(0), q_lat.stride(1),
+                       reinterpret_cast<const T*>(ckr.data_ptr()), ckr.stride(0),
+                       reinterpret_cast<const T*>(c_w.data_ptr()), inv_freq.data_ptr<float>(),
+                       positions.data_ptr<long>(), reinterpret_cast<T*>(k_cache.data_ptr()),
+                       slots.data_ptr<long>(), H, (int)dim, DR, R, (int)rot_dims,
+                       (int)interleaved, (float)eps);
+  });
+}
+
+// ---- gated parallel residual join
+void gated_residual_add(at::Tensor out, at::Tensor res, at::Tensor y1, at::Tensor g1, at::Tensor b1,
+                        const std::optional<at::Tensor>& y2, const std::optional<at::Tensor>& g2,
+                        const std::optional<at::Tensor>& b2) {
+  HY_GPU(res);
+  TORCH_CHECK(res.dim() == 2 && res.is_contiguous() && res.scalar_type() == at::kFloat, "res must be fp32 [rows, W]");
+  const long rows = res.size(0);
+  const int W = res.size(1);
+  if (rows == 0) return;
+  auto check_pair = [&](const at::Tensor& y, const at::Tensor& g, const at::Tensor& b) {
+    TORCH_CHECK(y.is_contiguous() && y.sizes() == res.sizes() && y.scalar_type() == out.scalar_type());
+    TORCH_CHECK(g.dim() == 2 && g.size(0) == rows && g.size(1) == W && g.stride(1) == 1 &&
+                g.scalar_type() == out.scalar_type());
+    TORCH_CHECK(b.scalar_type() == at::kFloat && b.is_contiguous() && b.numel() == W && b.is_cuda());
+  };
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == res.sizes());
+  check_pair(y1, g1, b1);
+  const bool two = y2.has_value();
+  TORCH_CHECK(g2.has_value() == two && b2.has_value() == two, "second sublayer needs y, g and b");
+  if (two) check_pair(*y2, *g2, *b2);
+  const long g2s = two ? g2->stride(0) : 0;
+  auto aligned = [](const at::Tensor& t) {
+    return reinterpret_cast<uintptr_t>(t.data_ptr()) % 16 == 0 && t.stride(0) % 8 == 0;
+  };
+  if (out.scalar_type() == at::kBFloat16 && W % 8 == 0 && aligned(g1) && (!two || aligned(*g2))) {
+    using bf = __hip_bfloat16;
+    const int grid = (int)std::min<long>((rows * (W / 8) + 255) / 256, 4096);
+    hipLaunchKernelGGL(gated_residual_add_vec_kernel, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<bf*>(out.data_ptr()), res.data_ptr<float>(),
+                       reinterpret_cast<const bf*>(y1.data_ptr()),
+                       reinterpret_cast<const bf*>(g1.data_ptr()), g1.stride(0), b1.data_ptr<float>(),
+                       two ? reinterpret_cast<const bf*>(y2->data_ptr()) : nullptr,
+                       two ? reinterpret_cast<const bf*>(g2->data_ptr()) : nullptr, g2s,
+                       two ? b2->data_ptr<float>() : nullptr, rows, W);
+    return;
+  }
+  hy_dispatch(out, "gated_residual_add", [&]<typename T>() {
+    const int grid = (int)std::min<long>((rows * W + 255) / 256, 4096);
+    hipLaunchKernelGGL(gated_residual_add_kernel<T>, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), res.data_ptr<float>(),
+                       reinterpret_cast<const T*>(y1.data_ptr()),
+                       reinterpret_cast<const T*>(g1.data_ptr()), g1.stride(0), b1.data_ptr<float>(),
+                       two ? reinterpret_cast<const T*>(y2->data_ptr()) : nullptr,
+                       two ? reinterpret_cast<const T*>(g2->data_ptr()) : nullptr, g2s,
+                       two ? b2->data_ptr<float>() : nullptr, rows, W);
+  });
+}
+
+void side_gate_mul(at::Tensor out, at::Tensor a, at::Tensor table, at::Tensor tokens, int64_t offset) {
+  HY_GPU(a);
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && out.is_contiguous() && out.sizes() == a.sizes());
+  const long rows = a.size(0);
+  const int d = a.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(table.dim() == 2 && table.is_contiguous() && offset >= 0 && offset + d <= table.size(1));
+  TORCH_CHECK(tokens.scalar_type() == at::kLong && tokens.is_contiguous() && tokens.numel() == rows);
+  TORCH_CHECK(table.scalar_type() == a.scalar_type() && out.scalar_type() == a.scalar_type());
+  hy_dispatch(a, "side_gate_mul", [&]<typename T>() {
+    const int grid = (int)std::min<long>((rows * d + 255) / 256, 4096);
+    hipLaunchKernelGGL(side_gate_mul_kernel<T>, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(a.data_ptr()),
+                       reinterpret_cast<const T*>(table.data_ptr()), table.stride(0),
+                       tokens.data_ptr<long>(), (int)offset, rows, d);
+  });
+}
+
+void sigmoid_topk(at::Tensor idx, at::Tensor w, at::Tensor logits, int64_t top) {
+  HY_GPU(logits);
+  TORCH_CHECK(logits.dim() == 2 && logits.is_contiguous() && logits.scalar_type() == at::kFloat,
+              "router logits must be fp32 [T, E]");
+  const long rows = logits.size(0);
+  const int E = logits.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(top >= 1 && top <= E && E <= 64 * 32, "top must be within 1..E, E at most 2048");
+  HY_I32(idx);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == rows && idx.size(1) == top);
+  TORCH_CHECK(w.scalar_type() == at::kFloat && w.is_contiguous() && w.sizes() == idx.sizes());
+  hipLaunchKernelGGL(sigmoid_topk_kernel, dim3((rows + 3) / 4), dim3(256), 0, hy_stream(),
+                     idx.data_ptr<int>(), w.data_ptr<float>(), logits.data_ptr<float>(), rows, E,
+                     (int)top);
+}
+
+struct MoeDims { long T; int top, W, F, E; };
+
+MoeDims moe_check(const at::Tensor& idx, int W, int F, int E) {
+  HY_I32(idx);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(1) >= 1, "idx must be [T, top]");
+  return MoeDims{idx.size(0), (int)idx.size(1), W, F, E};
+}
+
+void moe_gate_up_gemv(at::Tensor hmid, at::Tensor h, at::Tensor idx, at::Tensor w, at::Tensor gate_up) {
+  HY_GPU(h);
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && gate_up.dim() == 3 && gate_up.is_contiguous());
+  TORCH_CHECK(gate_up.size(1) % 2 == 0 && gate_up.size(2) == h.size(1));
+  const MoeDims m = moe_check(idx, h.size(1), gate_up.size(1) / 2, gate_up.size(0));
+  if (m.T == 0) return;
+  TORCH_CHECK(idx.size(0) == h.size(0));
+  TORCH_CHECK(w.scalar_type() == at::kFloat && w.is_contiguous() && w.sizes() == idx.sizes());
+  TORCH_CHECK(hmid.is_contiguous() && hmid.dim() == 2 && hmid.size(0) == m.T * m.top && hmid.size(1) == m.F);
+  TORCH_CHECK(hmid.scalar_type() == h.scalar_type() && gate_up.scalar_type() == h.scalar_type());
+  const size_t lds = sizeof(float) * (size_t)m.W;
+  const dim3 grid((m.F + 4 * kMoeRowsPerWave - 1) / (4 * kMoeRowsPerWave), m.T * m.top);
+  hy_dispatch(h, "moe_gate_up_gemv", [&]<typename T>() {
+    auto kern = moe_gate_up_gemv_kernel<T>;
+    allow_lds(kern, lds);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(hmid.data_ptr()),
+                       reinterpret_cast<const T*>(h.data_ptr()), idx.data_ptr<int>(),
+                       w.data_ptr<float>(), reinterpret_cast<const T*>(gate_up.data_ptr()), m.top,
+                       m.W, m.F, m.E);
+  });
+}
+
+void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor down) {
+  HY_GPU(hmid);
+  TORCH_CHECK(down.dim() == 3 && down.is_contiguous() && hmid.dim() == 2 && hmid.is_contiguous());
+  const MoeDims m = moe_check(idx, down.size(1), down.size(2), down.size(0));
+  if (m.T == 0) return;
+  TORCH_CHECK(hmid.size(0) == m.T * m.top && hmid.size(1) == m.F);
+  TORCH_CHECK(y.is_contiguous() && y.dim() == 2 && y.size(0) == m.T && y.size(1) == m.W);
+  TORCH_CHECK(y.scalar_type() == hmid.scalar_type() && down.scalar_type() == hmid.scalar_type());
+  const size_t lds = sizeof(float) * (size_t)m.top * m.F;
+  const dim3 grid((m.W + 4 * kMoeRowsPerWave - 1) / (4 * kMoeRowsPerWave), m.T);
+  hy_dispatch(hmid, "moe_down_gemv", [&]<typename T>() {
+    auto kern = moe_down_gemv_kernel<T>;
+    allow_lds(kern, lds);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(y.data_ptr()),
+                       reinterpret_cast<const T*>(hmid.data_ptr()), idx.data_ptr<int>(),
+                       reinterpret_cast<const T*>(down.data_ptr()), m.top, m.W, m.F, m.E);
   });
 }
 
@@ -368,10 +580,16 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("sandwich_norm_res32(Tensor(a!) x, Tensor(b!) residual, Tensor w_post, Tensor w_pre, float eps, float offset) -> ()");
   m.def("act_and_mul(Tensor(a!) out, Tensor input, bool gelu) -> ()");
   m.def("qknorm_vmix_cache(Tensor(a!) q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, Tensor? v_first, float lam, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slots, float eps) -> ()");
-  m.def("chunk_bias_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale) -> ()");
-  m.def("chunk_bias_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor v_cache, Tensor bias, Tensor block_tables, Tensor context_lens, int span, float scale) -> ()");
-  m.def("gla_recurrence(Tensor(a!) o, Tensor q, Tensor k, Tensor v, Tensor z, Tensor z_bias, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float tau) -> ()");
-  m.def("gla_out_norm_gate(Tensor(a!) out, Tensor o, Tensor weight, Tensor gate, float eps) -> ()");
+  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode) -> ()");
+  m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode) -> ()");
+  m.def("gla_recurrence(Tensor(a!) o, Tensor q, Tensor? k, Tensor v, Tensor z, Tensor z_bias, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float tau, Tensor? lower, bool q_silu, float q_scale) -> ()");
+  m.def("gla_out_norm_gate(Tensor(a!) out, Tensor o, Tensor weight, Tensor? gate, float eps) -> ()");
+  m.def("latent_rope_pack(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor ckr, Tensor c_w, Tensor inv_freq, Tensor positions, Tensor(b!) k_cache, Tensor slots, int dim, int rot_dims, bool interleaved, float eps) -> ()");
+  m.def("gated_residual_add(Tensor(a!) out, Tensor(b!) res, Tensor y1, Tensor g1, Tensor b1, Tensor? y2, Tensor? g2, Tensor? b2) -> ()");
+  m.def("side_gate_mul(Tensor(a!) out, Tensor a, Tensor table, Tensor tokens, int offset) -> ()");
+  m.def("sigmoid_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top) -> ()");
+  m.def("moe_gate_up_gemv(Tensor(a!) hmid, Tensor h, Tensor idx, Tensor w, Tensor gate_up) -> ()");
+  m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
@@ -379,8 +597,14 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("sandwich_norm_res32", &sandwich_norm_res32);
   m.impl("act_and_mul", &act_and_mul);
   m.impl("qknorm_vmix_cache", &qknorm_vmix_cache);
-  m.impl("chunk_bias_attn_prefill", &chunk_bias_attn_prefill);
-  m.impl("chunk_bias_attn_decode", &chunk_bias_attn_decode);
+  m.impl("paged_attn_prefill", &paged_attn_prefill);
+  m.impl("paged_attn_decode", &paged_attn_decode);
+  m.impl("latent_rope_pack", &latent_rope_pack);
+  m.impl("gated_residual_add", &gated_residual_add);
+  m.impl("side_gate_mul", &side_gate_mul);
+  m.impl("sigmoid_topk", &sigmoid_topk);
+  m.impl("moe_gate_up_gemv", &moe_gate_up_gemv);
+  m.impl("moe_down_gemv", &moe_down_gemv);
   m.impl("gla_recurrence", &gla_recurrence);
   m.impl("gla_out_norm_gate", &gla_out_norm_gate);
 }

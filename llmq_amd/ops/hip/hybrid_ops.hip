@@ -4,4 +4,5 @@
 // hybrid model builds nothing else.
 #include "elementwise.hip"
 #include "seqmix.hip"
+#include "latent_moe.hip"
 #include "hybrid_bindings.cpp"

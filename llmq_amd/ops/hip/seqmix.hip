@@ -1,7 +1,9 @@
 // Sequence-mixer kernels for hybrid decoders (gfx950): layers that keep the
-// residual stream in fp32, block-local ("chunked") attention with a learned
-// per-distance bias over the paged KV cache, and gated-linear-attention
-// recurrences over per-sequence fp32 state slots.
+// residual stream in fp32, attention over the paged KV cache under a
+// block-local ("chunked") or a sliding-window / causal mask, with an optional
+// learned per-distance bias and an optional per-head gate, and diagonal-decay
+// recurrences (gated linear attention, HGRN2) over per-sequence fp32 state
+// slots.
 //
 // Numerics contract shared by every kernel here: activations arrive in the
 // model dtype T (bf16 or fp32); norms, scores, softmax weights, decays and
@@ -15,11 +17,11 @@
 // out = rmsnorm(in) * (w + offset); TI/TO may differ (fp32 stream -> T).
 template <typename TI, typename TO>
 __global__ void rmsnorm_cast_kernel(TO* __restrict__ out, const TI* __restrict__ in,
-                                    const TO* __restrict__ weight, int hidden,
+                                    long in_stride, const TO* __restrict__ weight, int hidden,
                                     float eps, float offset) {
   __shared__ float red[4];
   const long row = blockIdx.x;
-  const TI* x = in + row * hidden;
+  const TI* x = in + row * in_stride;
   TO* o = out + row * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
@@ -223,6 +225,18 @@ __global__ void qknorm_vmix_cache_kernel(
 constexpr int kAttnQT = 16;
 constexpr int kAttnKT = 64;
 
+// Masks of the paged attention kernels. Block-local: query i sees key j iff
+// j <= i and both lie in the same span of `span` positions counted from 0.
+// Window: j <= i and i - j < span (a span beyond every context = causal).
+// Values sit in their own cache (row stride DV) or are the first DV channels
+// of the key rows (v_row = D, latent caches); a null bias adds nothing.
+constexpr int kMaskBlock = 0;
+constexpr int kMaskWindow = 1;
+
+DEVINL int mask_first_key(int pos, int span, int mode) {
+  return mode == kMaskBlock ? (pos / span) * span : max(0, pos - span + 1);
+}
+
 template <typename T, int NV>
 __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     T* __restrict__ out, long out_stride,
@@ -233,7 +247,8 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q,          // [B+1]
     const int* __restrict__ q_start,       // [B] position of a sequence's first query
-    int H, int G, int D, int DV, int block_size, int span, float scale) {
+    int H, int G, int D, int DV, int block_size, int span, float scale,
+    int v_row, int mask_mode) {
   extern __shared__ float smem[];
   const int b = blockIdx.z, h = blockIdx.y;
   const int row0 = cu_q[b];
@@ -266,7 +281,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     for (int n = 0; n < NV; ++n) acc[r][n] = 0.f;
   }
   const int* bt = block_tables + (long)b * bt_stride;
-  const int lo = (pos0 / span) * span;
+  const int lo = mask_first_key(pos0, span, mask_mode);
   for (int kt = lo; kt <= pos_last; kt += kAttnKT) {
     const int nk = min(kAttnKT, pos_last + 1 - kt);
     __syncthreads();
@@ -282,7 +297,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const int key = kt + jj;
       const long base = (((long)bt[key / block_size] * G + g) * block_size +
                          key % block_size);
-      Vs[jj * DV + d] = to_f32(v_cache[base * DV + d]);
+      Vs[jj * DV + d] = to_f32(v_cache[base * v_row + d]);
     }
     __syncthreads();
     // scores: lane = key, 4 rows at once
@@ -303,8 +318,9 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     for (int r = 0; r < 4; ++r) {
       const int i = pos0 + w * 4 + r;
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
-                       key / span == i / span;
-      const float sc = vis ? s[r] + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : -INFINITY;
+                       key >= mask_first_key(i, span, mask_mode);
+      const float sc = !vis ? -INFINITY
+          : bias ? s[r] + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : s[r];
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -382,7 +398,8 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const float* __restrict__ bias, int bias_len,   // [H, bias_len]
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
-    int H, int G, int D, int DV, int block_size, int span, float scale) {
+    int H, int G, int D, int DV, int block_size, int span, float scale,
+    int v_row, int mask_mode) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr int VG = DT / 2;             // 32-channel groups of V per thread
   const int b = blockIdx.z, h = blockIdx.y;
@@ -420,7 +437,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   for (int reg = 0; reg < 4; ++reg) {
     const int r = w * 16 + kgrp * 4 + reg;
     irow[reg] = r < rows ? pos0 + r : -1;       // -1: no key satisfies key <= irow
-    lorow[reg] = r < rows ? ((pos0 + r) / span) * span : 0;
+    lorow[reg] = r < rows ? mask_first_key(pos0 + r, span, mask_mode) : 0;
     m[reg] = -INFINITY;
     l[reg] = 0.f;
   }
@@ -429,12 +446,12 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   for (int dt = 0; dt < DT; ++dt) o[dt] = sm_f32x4{0.f, 0.f, 0.f, 0.f};
   const int wave_first = pos0 + w * 16;
   const int wave_last = min(pos_last, wave_first + 15);
-  const int wave_lo = (wave_first / span) * span;
+  const int wave_lo = mask_first_key(wave_first, span, mask_mode);
   const bool wave_rows = w * 16 < rows;
   const int* bt = block_tables + (long)b * bt_stride;
-  const float* bias_h = bias + (long)h * bias_len;
+  const float* bias_h = bias ? bias + (long)h * bias_len : nullptr;
   short* Pw = Ps + w * 2 * 16 * kMfmaKP;
-  const bool v_vec = (DV % 8) == 0;
+  const bool v_vec = (DV % 8) == 0 && (v_row % 8) == 0;
 
   // Staging map: thread = (key = tid/4, sub = tid%4) moves the 16-byte
   // granules sub*8 + 32*i of its key's K row and V row. The next tile's
@@ -459,7 +476,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       const int d8 = sub * 8 + 32 * i;
       sm_bf16x8 e = zero8;
       if (live && d8 < DV) {
-        const __hip_bfloat16* vr = v_cache + base * DV + d8;
+        const __hip_bfloat16* vr = v_cache + base * v_row + d8;
         if (v_vec) {
           e = *reinterpret_cast<const sm_bf16x8*>(vr);
         } else {
@@ -471,7 +488,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       vreg[i] = e;
     }
   };
-  const int kt0 = (pos0 / span) * span;
+  const int kt0 = mask_first_key(pos0, span, mask_mode);
   fetch(kt0);
   for (int kt = kt0; kt <= pos_last; kt += kMfmaKT) {
     __syncthreads();
@@ -489,7 +506,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     if (tid < 127) {
       // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)
       const int d = pos0 - kt - 63 + tid;
-      Bs[tid] = (d >= 0 && d < bias_len) ? bias_h[d] : 0.f;
+      Bs[tid] = (bias_h && d >= 0 && d < bias_len) ? bias_h[d] : 0.f;
     }
     __syncthreads();
     if (kt + kMfmaKT <= pos_last) fetch(kt + kMfmaKT);
@@ -603,7 +620,8 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     const float* __restrict__ bias, int bias_len,
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ context_lens,
-    int H, int G, int D, int DV, int block_size, int span, float scale) {
+    int H, int G, int D, int DV, int block_size, int span, float scale,
+    int v_row, int mask_mode) {
   extern __shared__ float smem[];
   const int h = blockIdx.x, b = blockIdx.y;
   const int g = h / (H / G);
@@ -616,7 +634,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     Qs[d] = to_f32(q[(long)b * q_stride + (long)h * D + d]) * scale;
   __syncthreads();
   const int i = context_lens[b] - 1;
-  const int lo = (i / span) * span;
+  const int lo = mask_first_key(i, span, mask_mode);
   const int* bt = block_tables + (long)b * bt_stride;
   float m = -INFINITY, l = 0.f, acc[NV];
 #pragma unroll
@@ -631,7 +649,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
       const T* kr = k_cache + base * D;
       float s = 0.f;
       for (int d = 0; d < D; ++d) s += Qs[d] * to_f32(kr[d]);
-      sc = s + bias[(long)h * bias_len + min(i - key, bias_len - 1)];
+      sc = bias ? s + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : s;
     }
     const float m_new = fmaxf(m, wave_reduce_max(sc));  // nk >= 1: finite
     const float corr = expf(m - m_new);
@@ -641,7 +659,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     for (int jj = 0; jj < nk; ++jj) {
       const float pj = __shfl(p, jj, WAVE);
       const long vb = __shfl(base, jj, WAVE);
-      const T* vr = v_cache + vb * DV;
+      const T* vr = v_cache + vb * v_row;
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         const int c = lane + 64 * n;
@@ -676,10 +694,15 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
   }
 }
 
-// ----------------------------------------------- gated linear attention ----
-// Per head, per sequence: S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t
-// with a_t = sigmoid(z_t + z_bias)^(1/tau) per key channel, state S in fp32
-// [D, DV] living in a per-sequence slot between steps.
+// ------------------------------------------- diagonal-decay recurrences ----
+// Per head, per sequence: S_t = diag(a_t) S_{t-1} + w_t v_t^T, o_t = S_t^T q_t,
+// state S in fp32 [D, DV] living in a per-sequence slot between steps. Two
+// forms of the decay a_t and the write strength w_t per key channel:
+//   gated linear attention (lower == null): a = sigmoid(z + z_bias)^(1/tau),
+//     w = k;
+//   HGRN2 (lower != null): a = l + (1 - l) * sigmoid(z + z_bias), w = 1 - a
+//     (no key is read).
+// q enters as q_scale * q, or q_scale * silu(q) with q_silu.
 //
 // Value columns evolve independently, so the grid splits DV: a workgroup owns
 // 32 columns of one (sequence, head), two per thread. Its 256 threads are 16 column pairs x 16 key
@@ -707,7 +730,9 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
     const int* __restrict__ cu,             // [B+1] row offsets
     const int* __restrict__ slots,          // [B]
     const int* __restrict__ fresh,          // [B]
-    int H, int D, int DV, float inv_tau, float q_scale) {
+    int H, int D, int DV, float inv_tau, float q_scale,
+    const float* __restrict__ lower,        // [H*D] or null
+    int q_silu) {
   constexpr int DP = 16 * DPL;          // padded key channels
   __shared__ __align__(16) float qs[kGlaTB * DP];
   __shared__ __align__(16) float ks[kGlaTB * DP];
@@ -747,7 +772,7 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
       if (tt < nt && d < D) {
         const long row = row0 + t0 + tt;
         rq[j] = to_f32(q[row * q_stride + (long)h * D + d]);
-        rk[j] = to_f32(k[row * k_stride + (long)h * D + d]);
+        if (k) rk[j] = to_f32(k[row * k_stride + (long)h * D + d]);
         rz[j] = to_f32(z[row * z_stride + (long)h * D + d]);
       }
     }
@@ -767,8 +792,20 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
     for (int j = 0; j < DPL; ++j) {
       const int idx = tid + 256 * j;
       const int d = idx % DP;
-      float av = 0.f;
-      if (d < D) {
+      float av = 0.f, kv = rk[j], qv = rq[j];
+      if (q_silu) {
+        if constexpr (std::is_same_v<T, float>) qv = qv / (1.0f + expf(-qv));
+        else qv = qv / (1.0f + __expf(-qv));
+      }
+      if (d < D && lower) {
+        const float zz = rz[j] + z_bias[h * D + d];
+        const float lo = lower[h * D + d];
+        float sg;
+        if constexpr (std::is_same_v<T, float>) sg = 1.0f / (1.0f + expf(-zz));
+        else sg = 1.0f / (1.0f + __expf(-zz));
+        av = lo + (1.0f - lo) * sg;
+        kv = 1.0f - av;
+      } else if (d < D) {
         const float zz = rz[j] + z_bias[h * D + d];
         // log sigmoid(zz) = min(zz, 0) - log1p(exp(-|zz|)); fp32 models take
         // the accurate library functions, bf16 models the hardware exp/log
@@ -781,8 +818,8 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
           av = __expf(ls * inv_tau);
         }
       }
-      qs[idx] = rq[j] * q_scale;
-      ks[idx] = rk[j];
+      qs[idx] = qv * q_scale;
+      ks[idx] = kv;
       as[idx] = av;
     }
     vs[tid] = rv[0];
@@ -853,7 +890,7 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
   }
 }
 
-// Per (token, head): out = rmsnorm_DV(o) * w * silu(gate), rounded to T.
+// Per (token, head): out = rmsnorm_DV(o) * w [* silu(gate)], rounded to T.
 // One wave per head, lanes over value channels.
 template <typename T>
 __global__ __launch_bounds__(256) void gla_out_norm_gate_kernel(
@@ -869,8 +906,11 @@ __global__ __launch_bounds__(256) void gla_out_norm_gate_kernel(
     ss = wave_reduce_sum(ss);
     const float inv = 1.0f / sqrtf(ss / DV + eps);
     for (int c = lane; c < DV; c += 64) {
-      const float gt = to_f32(gate[tok * g_stride + (long)h * DV + c]);
-      const float sg = gt / (1.0f + expf(-gt));
+      float sg = 1.f;
+      if (gate) {
+        const float gt = to_f32(gate[tok * g_stride + (long)h * DV + c]);
+        sg = gt / (1.0f + expf(-gt));
+      }
       out[tok * out_stride + (long)h * DV + c] =
           from_f32<T>(oh[c] * inv * to_f32(weight[c]) * sg);
     }

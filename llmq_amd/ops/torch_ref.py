@@ -377,3 +377,157 @@ def gla_out_norm_gate(o, weight, gate, eps, out_dtype):
     y = o * (1.0 / torch.sqrt(o.pow(2).mean(dim=-1, keepdim=True) + eps)) * weight.float()
     y = y.reshape(T, H * DV) * torch.nn.functional.silu(gate.float())
     return y.to(out_dtype)
+
+
+# ------------------------------------------- looped hybrid decoders (ref) --
+# Reference forms of the ops added for latent attention, lower-bounded
+# forget-gate recurrences, gated parallel residuals and expert mixtures.
+
+
+def _window_attend(qb, kc, vc, pos, window, scale):
+    """qb [n, H, D] at absolute positions pos [n]; kc [L, G, D], vc [L, G, DV]
+    cached keys/values of positions 0..L-1. Query i sees key j iff j <= i
+    and (window == 0 or i - j < window)."""
+    n, H, _ = qb.shape
+    G = kc.shape[1]
+    lo = max(0, int(pos[0]) - window + 1) if window else 0
+    kk = kc[lo:].float().repeat_interleave(H // G, dim=1)
+    vv = vc[lo:].float().repeat_interleave(H // G, dim=1)
+    j = torch.arange(lo, kc.shape[0], device=qb.device).view(1, -1)
+    i = pos.view(-1, 1)
+    vis = j <= i
+    if window:
+        vis = vis & (i - j < window)
+    scores = torch.einsum("ihd,jhd->hij", qb.float(), kk) * scale
+    scores = scores.masked_fill(~vis.unsqueeze(0), float("-inf"))
+    return torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), vv)
+
+
+def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, window, scale):
+    """Causal / sliding-window softmax attention of packed prompt portions
+    over the paged cache. v_cache None: a key row's first dv channels are
+    its value."""
+    T, H, _ = q.shape
+    out = q.new_empty(T, H, dv)
+    for b in range(len(q_start)):
+        s, e = int(cu_q[b]), int(cu_q[b + 1])
+        if e == s:
+            continue
+        p0 = int(q_start[b])
+        L = p0 + (e - s)
+        kc = _gather_seq(k_cache, block_tables[b], L)
+        vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
+        pos = torch.arange(p0, L, device=q.device)
+        out[s:e] = _window_attend(q[s:e], kc, vc, pos, window, scale).to(q.dtype)
+    return out
+
+
+def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, window, scale):
+    B, H, _ = q.shape
+    out = q.new_empty(B, H, dv)
+    for b in range(B):
+        L = int(context_lens[b])
+        kc = _gather_seq(k_cache, block_tables[b], L)
+        vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
+        pos = torch.tensor([L - 1], device=q.device)
+        out[b : b + 1] = _window_attend(q[b : b + 1], kc, vc, pos, window, scale).to(q.dtype)
+    return out
+
+
+def _rotate(x, positions, inv_freq, rot_dims, interleaved):
+    """x [T, ..., n] fp32: rotary positions on its first rot_dims channels."""
+    half = rot_dims // 2
+    ang = positions.float().view(-1, *([1] * (x.dim() - 2)), 1) * inv_freq.float()
+    cos, sin = torch.cos(ang), torch.sin(ang)
+    out = x.clone()
+    if interleaved:
+        u, v = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+        out[..., 0:rot_dims:2] = u * cos - v * sin
+        out[..., 1:rot_dims:2] = v * cos + u * sin
+    else:
+        u, v = x[..., :half], x[..., half:rot_dims]
+        out[..., :half] = u * cos - v * sin
+        out[..., half:rot_dims] = v * cos + u * sin
+    return out
+
+
+def latent_rope_pack(q, q_lat, ckr, c_w, inv_freq, positions, k_cache, slots, dim, rot_dims,
+                     interleaved, eps):
+    """q [T, H, dim+DR] (projection), q_lat [T, H, R] (its unrotated part
+    mapped into the latent), ckr [T, R+DR] (latent ‖ rotated key part).
+    Returns the packed query [T, H, R+DR] = q_lat ‖ rotate(q[..., dim:]) and
+    scatters rmsnorm(latent)*c_w ‖ rotate(key part) into the paged cache
+    [blocks, 1, bs, R+DR]."""
+    T, H, _ = q.shape
+    R = q_lat.shape[2]
+    q_rot = _rotate(q[..., dim:].float(), positions, inv_freq, rot_dims, interleaved)
+    out = torch.cat([q_lat.float(), q_rot], dim=-1).to(q.dtype)
+    c = rmsnorm_cast(ckr[:, :R], c_w, eps, 0.0, torch.float32)
+    k_rot = _rotate(ckr[:, R:].float(), positions, inv_freq, rot_dims, interleaved)
+    row = torch.cat([c, k_rot], dim=-1)
+    bs = k_cache.shape[2]
+    keep = slots >= 0
+    s = slots[keep].long()
+    k_cache[s // bs, 0, s % bs, :] = row[keep].to(k_cache.dtype)
+    return out
+
+
+def gated_recurrence(q, k, v, z, z_bias, state, cu, slots, fresh, tau, lower, q_silu, q_scale):
+    """The diagonal-decay recurrence S <- diag(a) S + w v^T, o = S^T q over
+    packed sequences. lower None: a = sigmoid(z + b)^(1/tau), w = k.
+    lower given: a = l + (1 - l) * sigmoid(z + b), w = 1 - a (k unused)."""
+    T, H, D = q.shape
+    o = torch.empty(T, H, v.shape[2], dtype=torch.float32, device=q.device)
+    zf = z.float() + z_bias.view(1, H, D)
+    if lower is None:
+        alpha = torch.exp(torch.nn.functional.logsigmoid(zf) / tau)
+        kf = k.float()
+    else:
+        lo = lower.float().view(1, H, D)
+        alpha = lo + (1.0 - lo) * torch.sigmoid(zf)
+        kf = 1.0 - alpha
+    qf = q.float()
+    if q_silu:
+        qf = torch.nn.functional.silu(qf)
+    qf = qf * q_scale
+    vf = v.float()
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        S = torch.zeros_like(state[slot]) if int(fresh[b]) else state[slot].clone()
+        for t in range(s, e):
+            S = alpha[t].unsqueeze(-1) * S + kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    return o
+
+
+def head_norm(o, weight, eps, out_dtype):
+    """Per-head RMSNorm over the value size of o [T, H, DV] fp32 -> [T, H*DV]."""
+    T, H, DV = o.shape
+    y = o * (1.0 / torch.sqrt(o.pow(2).mean(dim=-1, keepdim=True) + eps)) * weight.float()
+    return y.reshape(T, H * DV).to(out_dtype)
+
+
+def gated_residual_add(res, y1, g1, b1, y2, g2, b2, out_dtype):
+    """res (fp32, in place) += sigmoid(g1 + b1) * y1 [+ sigmoid(g2 + b2) * y2];
+    returns res rounded to out_dtype."""
+    add = torch.sigmoid(g1.float() + b1.float()) * y1.float()
+    if y2 is not None:
+        add = add + torch.sigmoid(g2.float() + b2.float()) * y2.float()
+    res.add_(add)
+    return res.to(out_dtype)
+
+
+def side_gate_mul(a, table, tokens, offset):
+    """gelu_tanh(a) * table[tokens, offset : offset + a.shape[1]] in a's dtype."""
+    e = table[tokens][:, offset : offset + a.shape[1]].float()
+    return (torch.nn.functional.gelu(a.float(), approximate="tanh") * e).to(a.dtype)
+
+
+def sigmoid_topk(logits, top):
+    """Router: scores = sigmoid(logits) (fp32); the `top` largest per row.
+    Returns (indices int32 [T, top], scores fp32 [T, top])."""
+    s = torch.sigmoid(logits.float())
+    w, idx = torch.topk(s, top, dim=-1)
+    return idx.to(torch.int32), w
