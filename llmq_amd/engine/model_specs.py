@@ -487,7 +487,7 @@ class KosalornSpec:
         total += self.vocab_size * self.side_dim * len(self.layers)
         for ls in self.layers:
             m = ls.mixer
-            total += 1 + 2 * (w * w + w)
+            total += 1 + (2 if (ls.ff or ls.moe) else 1) * (w * w + w)
             if m.kind == "hgrn2":
                 nk, nv = m.heads * m.dim, m.heads * m.vdim
                 total += 2 * nk * w + 2 * nk + nv * w + m.vdim + w * nv
