@@ -44,7 +44,8 @@ def compare_hybrid(args) -> None:
     models = args.compare_models.split(",")
     batch, prompt_len = min(args.batch, 64), args.prompt_len
     if not use_gpu:
-        models, batch, prompt_len = ["tiny-kakovik", "tiny-llama"], 4, 48
+        tiny = ["tiny-kosalorn"] if args.compare_kosalorn else []
+        models, batch, prompt_len = tiny + ["tiny-kakovik", "tiny-llama"], 4, 48
     for name in models:
         engine = LLMEngine(EngineConfig(
             model=name, max_num_seqs=batch,
@@ -125,9 +126,17 @@ def main() -> None:
                         help="instead of the headline workload: prefill and decode "
                         "throughput of the Kakovik hybrid presets beside the Llama "
                         "presets of equal layer sizes (one JSON line per model)")
-    parser.add_argument("--compare-models", default="kakovik-1b,llama-3.2-1b,kakovik-3b,llama-3.2-3b")
+    parser.add_argument("--compare-models", default=None)
+    parser.add_argument("--compare-kosalorn", action="store_true",
+                        help="the same comparison for the Kosalorn looped-hybrid presets "
+                        "(latent attention, HGRN2, expert mixtures) beside the Kakovik "
+                        "and Llama presets of equal layer sizes")
     args = parser.parse_args()
-    if args.compare_hybrid:
+    if args.compare_models is None:
+        args.compare_models = (
+            "kosalorn-1b,kosalorn-1b-moe,kakovik-1b,llama-3.2-1b,kosalorn-3b,kakovik-3b,llama-3.2-3b"
+            if args.compare_kosalorn else "kakovik-1b,llama-3.2-1b,kakovik-3b,llama-3.2-3b")
+    if args.compare_hybrid or args.compare_kosalorn:
         compare_hybrid(args)
         return
 

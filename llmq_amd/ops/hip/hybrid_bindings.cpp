@@ -244,9 +244,9 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
     const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H, B);
     using bf = __hip_bfloat16;
     auto launch = [&]<int KS, int DT>() {
-      // K tile, V^T tile (all DT*16 channel rows), P hi/lo per wave, bias slice
+      // K tile, V^T tile (the channel tiles in use), P hi/lo per wave, bias slice
       const size_t lds = sizeof(short) * ((size_t)kMfmaKT * (ksn * 32 + 8) +
-                                          (size_t)DT * 16 * kMfmaKP +
+                                          (size_t)dtn * 16 * kMfmaKP +
                                           (size_t)4 * 2 * 16 * kMfmaKP) + 128 * sizeof(float);
       auto kern = chunk_bias_attn_prefill_mfma_kernel<KS, DT>;
       allow_lds(kern, lds);

@@ -376,7 +376,9 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
 //
 // Workgroup = 64 query rows x 1 head, one wave per 16 rows. Per 64-key tile:
 // K is staged row-major [key][D] and V transposed [channel][key] in LDS, so
-// every MFMA operand is one 16-byte LDS read. S = Q K^T and O += P V run on
+// every MFMA operand is one 16-byte LDS read. When values are the first
+// channels of the key rows (v_cache == k_cache) the V tile is filled from the
+// K granules already in registers: nothing is fetched twice. S = Q K^T and O += P V run on
 // v_mfma_f32_16x16x32_bf16 (A: row = lane%16, k = 8*(lane/16)..+7; C: rows
 // 4*(lane/16)+reg, column lane%16), which puts a query row's scores and its
 // output in the same registers of the same lanes: the online-softmax rescale
@@ -412,10 +414,11 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   const int pos_last = pos0 + rows - 1;
   const int g = h / (H / G);
   const int ksn = (D + 31) / 32, dtn = (DV + 15) / 16;
+  const bool v_alias = v_cache == k_cache;             // values = prefix of the key rows
   const int Dp = ksn * 32, DS = Dp + 8;
   short* Ks = reinterpret_cast<short*>(smem_raw);     // [KT][DS]
-  short* Vt = Ks + kMfmaKT * DS;                      // [DT*16][KP]
-  short* Ps = Vt + DT * 16 * kMfmaKP;                 // [4 waves][hi, lo][16][KP]
+  short* Vt = Ks + kMfmaKT * DS;                      // [dtn*16][KP]
+  short* Ps = Vt + dtn * 16 * kMfmaKP;                // [4 waves][hi, lo][16][KP]
   float* Bs = reinterpret_cast<float*>(Ps + 4 * 2 * 16 * kMfmaKP);  // [128] bias slice
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int col = lane & 15, kgrp = lane >> 4;
@@ -475,7 +478,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     for (int i = 0; i < VG; ++i) {
       const int d8 = sub * 8 + 32 * i;
       sm_bf16x8 e = zero8;
-      if (live && d8 < DV) {
+      if (!v_alias && live && d8 < DV) {
         const __hip_bfloat16* vr = v_cache + base * v_row + d8;
         if (v_vec) {
           e = *reinterpret_cast<const sm_bf16x8*>(vr);
@@ -500,8 +503,11 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 #pragma unroll
     for (int i = 0; i < VG; ++i) {
       const int d8 = sub * 8 + 32 * i;
+      if (d8 < dtn * 16) {
+        const sm_bf16x8 e = v_alias ? kreg[i] : vreg[i];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) Vt[(d8 + j) * kMfmaKP + skey] = vreg[i][j];
+        for (int j = 0; j < 8; ++j) Vt[(d8 + j) * kMfmaKP + skey] = e[j];
+      }
     }
     if (tid < 127) {
       // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)

@@ -102,3 +102,17 @@ def test_bench_compare_hybrid_option():
     assert [l["family"] for l in lines] == ["kakovik", "llama"]
     for l in lines:
         assert l["prefill_tokens_per_sec"] > 0 and l["decode_tokens_per_sec"] > 0
+
+
+@pytest.mark.timeout(300)
+def test_bench_compare_kosalorn_option():
+    """--compare-kosalorn adds the looped-hybrid preset to the same comparison."""
+    proc = subprocess.run(
+        [sys.executable, "bench.py", "--compare-kosalorn", "--steps", "3", "--warmup", "1"],
+        capture_output=True, text=True, cwd=REPO, timeout=280,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    lines = [json.loads(l) for l in proc.stdout.splitlines() if l.startswith("{")]
+    assert [l["family"] for l in lines] == ["kosalorn", "kakovik", "llama"]
+    for l in lines:
+        assert l["prefill_tokens_per_sec"] > 0 and l["decode_tokens_per_sec"] > 0
