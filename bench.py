@@ -70,8 +70,13 @@ def compare_hybrid(args) -> None:
                 engine.step()
             sync()
 
+        def note(what):
+            print(f"[bench] {name}: {what}", file=sys.stderr, flush=True)
+
+        note("engine ready, warm prefill")
         load("warm")            # untimed pass: allocator, GEMM selection
         prefill_all()
+        note("timed prefill")
         for i in range(batch):
             engine.abort_request(f"warm-{i}")
         load("run")
@@ -79,6 +84,7 @@ def compare_hybrid(args) -> None:
         t0 = time.perf_counter()
         prefill_all()
         prefill_s = time.perf_counter() - t0
+        note("decode")
         for _ in range(args.warmup):
             engine.step()
         sync()

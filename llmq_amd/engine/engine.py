@@ -196,7 +196,7 @@ class LLMEngine:
         overlap_env = os.environ.get("LLMQ_OVERLAP_MIXED")
         overlap_default = not (
             self.spec.family == "gemma2" and self.spec.head_dim == 128
-        )
+        ) and getattr(model_cls, "overlap_mixed", True)
         self._overlap_mixed = (
             self.device.type == "cuda"
             and tp == 1

@@ -78,6 +78,11 @@ class KosalornLM:
     ext_groups = ("hybrid",)
     #: prompt portions attend through the block table (no gathered copy)
     paged_prefill = True
+    #: mixed steps run their decode and prefill segments one after the other:
+    #: this family's projection shapes select hipBLASLt stream-k GEMMs, whose
+    #: workgroups wait on each other and must not share the chip with a second
+    #: stream's kernels (LLMQ_OVERLAP_MIXED=1 forces the overlap back on)
+    overlap_mixed = False
 
     def __init__(self, spec: KosalornSpec, device: torch.device, dtype: torch.dtype,
                  tp_rank: int = 0, tp_size: int = 1):

@@ -595,6 +595,10 @@ def sigmoid_topk(logits, top: int):
 # rows (token, expert) pairs up to which the expert mixture runs as
 # per-row matrix-vector kernels (no host sync, graph-capturable)
 MOE_GEMV_MAX_ROWS = 64
+# within the matrix-vector form: from this many rows on (and up to the LDS
+# row list's size) rows are grouped by expert inside the kernel
+MOE_GROUP_MIN_ROWS = 16
+MOE_GROUP_MAX_ROWS = 2048
 
 
 def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False) -> torch.Tensor:
@@ -611,6 +615,14 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False) -> torch.Tens
         _use_hybrid(h)
         F_ = down.shape[2]
         hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
+        if MOE_GROUP_MIN_ROWS <= T * top <= MOE_GROUP_MAX_ROWS and \
+                max(h.shape[1], F_) * h.element_size() * 8 <= (128 << 10):
+            # enough rows that experts repeat: grouped by expert inside the
+            # kernel, a weight row is read once per 8 rows of its expert
+            _HY.moe_expert_gemv(hmid, h, idx, w, gate_up, True)
+            yk = torch.empty(T * top, h.shape[1], dtype=h.dtype, device=h.device)
+            _HY.moe_expert_gemv(yk, hmid, idx, None, down, False)
+            return yk.view(T, top, -1).float().sum(dim=1).to(h.dtype)
         _HY.moe_gate_up_gemv(hmid, h, idx, w, gate_up)
         y = torch.empty_like(h)
         _HY.moe_down_gemv(y, hmid, idx, down)

@@ -296,12 +296,17 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
   HY_I32(context_lens);
   const int B = q.size(0);
   TORCH_CHECK(context_lens.numel() == B && block_tables.size(0) == B);
-  const size_t lds = sizeof(float) * ((size_t)a.D + 4 * 64 + 8 + 4 * (size_t)a.DV);
-  hy_dispatch(q, "chunk_bias_attn_decode", [&]<typename T>() {
+  // query heads per workgroup: as many of one kv head's as divide evenly
+  const int per_kv = a.H / a.G;
+  const int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 2 == 0 ? 2 : 1;
+  const size_t lds = sizeof(float) * ((size_t)hpw * ((a.D + 3) & ~3) + 8 * hpw +
+                                      4 * (size_t)hpw * a.DV);
+  hy_dispatch(q, "paged_attn_decode", [&]<typename T>() {
     dispatch_nv(a.DV, [&]<int NV>() {
-      auto kern = chunk_bias_attn_decode_kernel<T, NV>;
+      auto launch = [&]<int HPW>() {
+      auto kern = chunk_bias_attn_decode_kernel<T, NV, HPW>;
       allow_lds(kern, lds);
-      hipLaunchKernelGGL(kern, dim3(a.H, B), dim3(256), lds, hy_stream(),
+      hipLaunchKernelGGL(kern, dim3(a.H / HPW, B), dim3(256), lds, hy_stream(),
                          reinterpret_cast<T*>(out.data_ptr()), out.stride(0),
                          reinterpret_cast<const T*>(q.data_ptr()), q.stride(0),
                          gate.has_value() ? reinterpret_cast<const T*>(gate->data_ptr()) : nullptr,
@@ -311,6 +316,11 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          context_lens.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs, (int)span,
                          (float)scale, a.v_row, (int)mask_mode);
+      };
+      if (hpw == 8) launch.template operator()<8>();
+      else if (hpw == 4) launch.template operator()<4>();
+      else if (hpw == 2) launch.template operator()<2>();
+      else launch.template operator()<1>();
     });
   });
 }
@@ -573,6 +583,45 @@ void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor dow
   });
 }
 
+// Expert mixture grouped by expert, no host sync. gate_up: in = h [T, W],
+// out = hmid [T*top, F]; else: in = hmid [T*top, F], out = yk [T*top, W].
+void moe_expert_gemv(at::Tensor out, at::Tensor in, at::Tensor idx, const std::optional<at::Tensor>& w,
+                     at::Tensor weight, bool gate_up) {
+  HY_GPU(in);
+  HY_I32(idx);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(1) >= 1, "idx must be [T, top]");
+  const long rows = idx.numel();
+  const int top = idx.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(rows <= kMoeMaxRows, "grouped expert kernel handles at most ", kMoeMaxRows, " rows");
+  TORCH_CHECK(weight.dim() == 3 && weight.is_contiguous() && in.dim() == 2 && in.is_contiguous() &&
+              out.dim() == 2 && out.is_contiguous());
+  const int E = weight.size(0), K = weight.size(2);
+  const int N = gate_up ? weight.size(1) / 2 : weight.size(1);
+  TORCH_CHECK(in.size(1) == K && out.size(0) == rows && out.size(1) == N);
+  TORCH_CHECK(in.size(0) == (gate_up ? idx.size(0) : rows));
+  TORCH_CHECK(in.scalar_type() == out.scalar_type() && weight.scalar_type() == out.scalar_type());
+  const float* wp = nullptr;
+  if (gate_up) {
+    TORCH_CHECK(weight.size(1) % 2 == 0 && w.has_value() && w->scalar_type() == at::kFloat &&
+                w->is_contiguous() && w->numel() == rows && w->is_cuda());
+    wp = w->data_ptr<float>();
+  }
+  const dim3 grid((N + 4 * kMoeFPW - 1) / (4 * kMoeFPW), E);
+  hy_dispatch(in, "moe_expert_gemv", [&]<typename T>() {
+    const size_t lds = sizeof(int) * kMoeMaxRows + sizeof(T) * (size_t)kMoeTB * K;
+    auto launch = [&]<bool GU>() {
+      auto kern = moe_expert_gemv_kernel<T, GU>;
+      allow_lds(kern, lds);
+      hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
+                         reinterpret_cast<const T*>(in.data_ptr()), idx.data_ptr<int>(), wp,
+                         reinterpret_cast<const T*>(weight.data_ptr()), (int)rows, top, K, N);
+    };
+    if (gate_up) launch.template operator()<true>();
+    else launch.template operator()<false>();
+  });
+}
+
 }  // namespace
 
 TORCH_LIBRARY(llmq_amd_hybrid, m) {
@@ -590,6 +639,7 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("sigmoid_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top) -> ()");
   m.def("moe_gate_up_gemv(Tensor(a!) hmid, Tensor h, Tensor idx, Tensor w, Tensor gate_up) -> ()");
   m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down) -> ()");
+  m.def("moe_expert_gemv(Tensor(a!) out, Tensor input, Tensor idx, Tensor? w, Tensor weight, bool gate_up) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
@@ -605,6 +655,7 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("sigmoid_topk", &sigmoid_topk);
   m.impl("moe_gate_up_gemv", &moe_gate_up_gemv);
   m.impl("moe_down_gemv", &moe_down_gemv);
+  m.impl("moe_expert_gemv", &moe_expert_gemv);
   m.impl("gla_recurrence", &gla_recurrence);
   m.impl("gla_out_norm_gate", &gla_out_norm_gate);
 }

@@ -291,3 +291,110 @@ __global__ __launch_bounds__(256) void moe_down_gemv_kernel(
     if (lane == 0) y[t * W + c] = from_f32<T>(acc);
   }
 }
+
+// --------------------------------- expert mixture, grouped by expert ------
+// The sync-free form for decode batches: one workgroup per (expert, tile of
+// output features) collects the rows routed to its expert from idx (in LDS,
+// no host round trip, no sort) and runs them in chunks of kMoeTB rows, so a
+// weight row is read once per chunk instead of once per row. Inputs of a
+// chunk sit in LDS in the model dtype; accumulation is fp32.
+//   GATE_UP: weight [E, 2F, K], x[r] = round(w[r] * h[r / top]), out hmid[r, f] =
+//            silu(gate_f . x) * (up_f . x)
+//   else   : weight [E, N, K], x[r] = in[r], out[r, n] = weight_n . x
+constexpr int kMoeTB = 8;        // rows per chunk
+constexpr int kMoeFPW = 2;       // output features per wave and pass
+constexpr int kMoeMaxRows = 2048;
+
+template <typename T, bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_expert_gemv_kernel(
+    T* __restrict__ out, const T* __restrict__ in, const int* __restrict__ idx,
+    const float* __restrict__ w, const T* __restrict__ weight, int rows, int top, int K, int N) {
+  extern __shared__ __align__(16) unsigned char moe_smem[];
+  __shared__ int count;
+  int* list = reinterpret_cast<int*>(moe_smem);                 // [kMoeMaxRows]
+  T* xs = reinterpret_cast<T*>(moe_smem + sizeof(int) * kMoeMaxRows);   // [kMoeTB][K]
+  const int e = blockIdx.y;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  if (tid == 0) count = 0;
+  __syncthreads();
+  for (int r = tid; r < rows; r += 256)
+    if (idx[r] == e) list[atomicAdd(&count, 1)] = r;
+  __syncthreads();
+  const int n = count;
+  if (n == 0) return;
+  constexpr int VE = Vec8<T>::kElems;
+  const int n0 = (blockIdx.x * 4 + wv) * kMoeFPW;
+  const T* we = weight + (long)e * (GATE_UP ? 2 : 1) * N * K;
+  for (int c0 = 0; c0 < n; c0 += kMoeTB) {
+    const int nt = min(kMoeTB, n - c0);
+    __syncthreads();
+    for (int i = tid; i < kMoeTB * K; i += 256) {
+      const int tt = i / K, k = i % K;
+      float v = 0.f;
+      if (tt < nt) {
+        const int r = list[c0 + tt];
+        v = GATE_UP ? to_f32(from_f32<T>(w[r] * to_f32(in[(long)(r / top) * K + k])))
+                    : to_f32(in[(long)r * K + k]);
+      }
+      xs[i] = from_f32<T>(v);
+    }
+    __syncthreads();
+    for (int f = n0; f < min(N, n0 + kMoeFPW); ++f) {
+      float a0[kMoeTB], a1[kMoeTB];
+#pragma unroll
+      for (int tt = 0; tt < kMoeTB; ++tt) a0[tt] = a1[tt] = 0.f;
+      const T* r0 = we + (long)f * K;
+      const T* r1 = we + (long)(N + f) * K;       // the up row (GATE_UP only)
+      if (K % VE == 0) {
+        for (int k = lane * VE; k < K; k += 64 * VE) {
+          const Vec8<T> g8 = load16(r0 + k);
+          Vec8<T> u8 = g8;
+          if (GATE_UP) u8 = load16(r1 + k);
+#pragma unroll
+          for (int tt = 0; tt < kMoeTB; ++tt) {
+            const Vec8<T> x8 = load16(xs + tt * K + k);
+#pragma unroll
+            for (int j = 0; j < VE; ++j) {
+              const float xv = to_f32(x8.data[j]);
+              a0[tt] += to_f32(g8.data[j]) * xv;
+              if (GATE_UP) a1[tt] += to_f32(u8.data[j]) * xv;
+            }
+          }
+        }
+      } else {
+        for (int k = lane; k < K; k += 64) {
+          const float gv = to_f32(r0[k]);
+          const float uv = GATE_UP ? to_f32(r1[k]) : 0.f;
+#pragma unroll
+          for (int tt = 0; tt < kMoeTB; ++tt) {
+            const float xv = to_f32(xs[tt * K + k]);
+            a0[tt] += gv * xv;
+            if (GATE_UP) a1[tt] += uv * xv;
+          }
+        }
+      }
+#pragma unroll
+      for (int tt = 0; tt < kMoeTB; ++tt) {
+        a0[tt] = wave_reduce_sum(a0[tt]);
+        if (GATE_UP) a1[tt] = wave_reduce_sum(a1[tt]);
+      }
+      if (lane < nt) {
+        float g = 0.f, u = 0.f;
+#pragma unroll
+        for (int tt = 0; tt < kMoeTB; ++tt)
+          if (tt == lane) {
+            g = a0[tt];
+            u = a1[tt];
+          }
+        const long r = list[c0 + lane];
+        g = to_f32(from_f32<T>(g));
+        if (GATE_UP) {
+          u = to_f32(from_f32<T>(u));
+          out[r * N + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+        } else {
+          out[r * N + f] = from_f32<T>(g);
+        }
+      }
+    }
+  }
+}

@@ -614,10 +614,15 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 }
 
 // ------------------------------------------------ attention: single tokens --
-// One workgroup per (sequence, head); the query is the sequence's newest
-// token (position ctx-1). Waves take key tiles of 64 round-robin, each with
-// its own online softmax; partials merge through LDS.
-template <typename T, int NV>
+// One workgroup per (sequence, group of HPW query heads that share a kv
+// head); the query is the sequence's newest token (position ctx-1). Waves
+// take key tiles of 64 round-robin, each with its own online softmax per
+// head; partials merge through LDS. A lane owns one key of the tile: it reads
+// that key's row once (16-byte loads when the row allows) and scores all HPW
+// heads against it; in the PV phase a lane owns value channels and every
+// value it reads feeds all HPW heads. With one kv head for all query heads
+// (latent caches) the cache is read H / HPW times instead of H times.
+template <typename T, int NV, int HPW>
 __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     T* __restrict__ out, long out_stride,
     const T* __restrict__ q, long q_stride,
@@ -628,75 +633,127 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     const int* __restrict__ context_lens,
     int H, int G, int D, int DV, int block_size, int span, float scale,
     int v_row, int mask_mode) {
-  extern __shared__ float smem[];
-  const int h = blockIdx.x, b = blockIdx.y;
-  const int g = h / (H / G);
+  extern __shared__ __align__(16) float smem[];
+  const int h0 = blockIdx.x * HPW, b = blockIdx.y;
+  const int g = h0 / (H / G);
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  float* Qs = smem;                    // [D]
-  float* Ps = Qs + D;                  // [4][64]
-  float* Ms = Ps + 4 * 64;             // [4] max, [4] sum
-  float* As = Ms + 8;                  // [4][DV]
-  for (int d = tid; d < D; d += 256)
-    Qs[d] = to_f32(q[(long)b * q_stride + (long)h * D + d]) * scale;
+  const int Dq = (D + 3) & ~3;         // padded so float4 reads stay in a head's row
+  float* Qs = smem;                    // [HPW][Dq]
+  float* Ms = Qs + HPW * Dq;           // [4][HPW] max, [4][HPW] sum
+  float* As = Ms + 8 * HPW;            // [4][HPW][DV]
+  for (int idx = tid; idx < HPW * Dq; idx += 256) {
+    const int hh = idx / Dq, d = idx % Dq;
+    Qs[idx] = d < D ? to_f32(q[(long)b * q_stride + (long)(h0 + hh) * D + d]) * scale : 0.f;
+  }
   __syncthreads();
   const int i = context_lens[b] - 1;
   const int lo = mask_first_key(i, span, mask_mode);
   const int* bt = block_tables + (long)b * bt_stride;
-  float m = -INFINITY, l = 0.f, acc[NV];
+  constexpr int VE = Vec8<T>::kElems;
+  const bool k_vec = (D % VE) == 0;
+  float m[HPW], l[HPW], acc[HPW][NV];
 #pragma unroll
-  for (int n = 0; n < NV; ++n) acc[n] = 0.f;
+  for (int hh = 0; hh < HPW; ++hh) {
+    m[hh] = -INFINITY;
+    l[hh] = 0.f;
+#pragma unroll
+    for (int n = 0; n < NV; ++n) acc[hh][n] = 0.f;
+  }
   for (int kt = lo + w * 64; kt <= i; kt += 4 * 64) {
     const int nk = min(64, i + 1 - kt);
     const int key = kt + lane;
     long base = 0;
-    float sc = -INFINITY;
+    float sc[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) sc[hh] = -INFINITY;
     if (lane < nk) {
       base = ((long)bt[key / block_size] * G + g) * block_size + key % block_size;
       const T* kr = k_cache + base * D;
-      float s = 0.f;
-      for (int d = 0; d < D; ++d) s += Qs[d] * to_f32(kr[d]);
-      sc = bias ? s + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : s;
+      float s[HPW];
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) s[hh] = 0.f;
+      if (k_vec) {
+        for (int d = 0; d < D; d += VE) {
+          const Vec8<T> kv = load16(kr + d);
+          float kf[VE];
+#pragma unroll
+          for (int j = 0; j < VE; ++j) kf[j] = to_f32(kv.data[j]);
+#pragma unroll
+          for (int hh = 0; hh < HPW; ++hh) {
+#pragma unroll
+            for (int j = 0; j < VE; j += 4) {
+              const float4 q4 = *reinterpret_cast<const float4*>(Qs + hh * Dq + d + j);
+              s[hh] += q4.x * kf[j] + q4.y * kf[j + 1] + q4.z * kf[j + 2] + q4.w * kf[j + 3];
+            }
+          }
+        }
+      } else {
+        for (int d = 0; d < D; ++d) {
+          const float kd = to_f32(kr[d]);
+#pragma unroll
+          for (int hh = 0; hh < HPW; ++hh) s[hh] += Qs[hh * Dq + d] * kd;
+        }
+      }
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh)
+        sc[hh] = bias ? s[hh] + bias[(long)(h0 + hh) * bias_len + min(i - key, bias_len - 1)]
+                      : s[hh];
     }
-    const float m_new = fmaxf(m, wave_reduce_max(sc));  // nk >= 1: finite
-    const float corr = expf(m - m_new);
-    const float p = lane < nk ? expf(sc - m_new) : 0.f;
-    l = l * corr + wave_reduce_sum(p);
-    m = m_new;
+    float p[HPW];
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      const float m_new = fmaxf(m[hh], wave_reduce_max(sc[hh]));  // nk >= 1: finite
+      const float corr = expf(m[hh] - m_new);
+      p[hh] = lane < nk ? expf(sc[hh] - m_new) : 0.f;
+      l[hh] = l[hh] * corr + wave_reduce_sum(p[hh]);
+      m[hh] = m_new;
+#pragma unroll
+      for (int n = 0; n < NV; ++n) acc[hh][n] *= corr;
+    }
     for (int jj = 0; jj < nk; ++jj) {
-      const float pj = __shfl(p, jj, WAVE);
       const long vb = __shfl(base, jj, WAVE);
       const T* vr = v_cache + vb * v_row;
+      float vv[NV];
 #pragma unroll
       for (int n = 0; n < NV; ++n) {
         const int c = lane + 64 * n;
-        if (jj == 0) acc[n] *= corr;
-        if (c < DV) acc[n] += pj * to_f32(vr[c]);
+        vv[n] = c < DV ? to_f32(vr[c]) : 0.f;
+      }
+#pragma unroll
+      for (int hh = 0; hh < HPW; ++hh) {
+        const float pj = __shfl(p[hh], jj, WAVE);
+#pragma unroll
+        for (int n = 0; n < NV; ++n) acc[hh][n] += pj * vv[n];
       }
     }
   }
-  if (lane == 0) {
-    Ms[w] = m;
-    Ms[4 + w] = l;
-  }
 #pragma unroll
-  for (int n = 0; n < NV; ++n) {
-    const int c = lane + 64 * n;
-    if (c < DV) As[w * DV + c] = acc[n];
+  for (int hh = 0; hh < HPW; ++hh) {
+    if (lane == 0) {
+      Ms[w * HPW + hh] = m[hh];
+      Ms[(4 + w) * HPW + hh] = l[hh];
+    }
+#pragma unroll
+    for (int n = 0; n < NV; ++n) {
+      const int c = lane + 64 * n;
+      if (c < DV) As[((long)w * HPW + hh) * DV + c] = acc[hh][n];
+    }
   }
   __syncthreads();
-  float mm = fmaxf(fmaxf(Ms[0], Ms[1]), fmaxf(Ms[2], Ms[3]));
-  float f[4], ll = 0.f;
+  for (int idx = tid; idx < HPW * DV; idx += 256) {
+    const int hh = idx / DV, c = idx % DV;
+    const float mm = fmaxf(fmaxf(Ms[hh], Ms[HPW + hh]), fmaxf(Ms[2 * HPW + hh], Ms[3 * HPW + hh]));
+    float a = 0.f, ll = 0.f;
 #pragma unroll
-  for (int ww = 0; ww < 4; ++ww) {
-    f[ww] = Ms[ww] > -INFINITY ? expf(Ms[ww] - mm) : 0.f;
-    ll += Ms[4 + ww] * f[ww];
-  }
-  float gs = 1.f;
-  if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[(long)b * g_stride + h])));
-  for (int c = tid; c < DV; c += 256) {
-    const float a = As[c] * f[0] + As[DV + c] * f[1] + As[2 * DV + c] * f[2] +
-                    As[3 * DV + c] * f[3];
-    out[(long)b * out_stride + (long)h * DV + c] = from_f32<T>(a * gs / ll);
+    for (int ww = 0; ww < 4; ++ww) {
+      const float mw = Ms[ww * HPW + hh];
+      const float f = mw > -INFINITY ? expf(mw - mm) : 0.f;
+      ll += Ms[(4 + ww) * HPW + hh] * f;
+      a += As[((long)ww * HPW + hh) * DV + c] * f;
+    }
+    float gs = 1.f;
+    if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[(long)b * g_stride + h0 + hh])));
+    out[(long)b * out_stride + (long)(h0 + hh) * DV + c] = from_f32<T>(a * gs / ll);
   }
 }
 
