@@ -299,14 +299,14 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
   // query heads per workgroup: as many of one kv head's as divide evenly
   const int per_kv = a.H / a.G;
   const int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 2 == 0 ? 2 : 1;
-  const size_t lds = sizeof(float) * ((size_t)hpw * ((a.D + 3) & ~3) + 8 * hpw +
-                                      4 * (size_t)hpw * a.DV);
+  const size_t lds = sizeof(float) * ((size_t)hpw * ((a.D + 3) & ~3) + 2 * kDecWaves * hpw +
+                                      (size_t)kDecWaves * hpw * a.DV);
   hy_dispatch(q, "paged_attn_decode", [&]<typename T>() {
     dispatch_nv(a.DV, [&]<int NV>() {
       auto launch = [&]<int HPW>() {
       auto kern = chunk_bias_attn_decode_kernel<T, NV, HPW>;
       allow_lds(kern, lds);
-      hipLaunchKernelGGL(kern, dim3(a.H / HPW, B), dim3(256), lds, hy_stream(),
+      hipLaunchKernelGGL(kern, dim3(a.H / HPW, B), dim3(64 * kDecWaves), lds, hy_stream(),
                          reinterpret_cast<T*>(out.data_ptr()), out.stride(0),
                          reinterpret_cast<const T*>(q.data_ptr()), q.stride(0),
                          gate.has_value() ? reinterpret_cast<const T*>(gate->data_ptr()) : nullptr,

@@ -621,9 +621,13 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 // that key's row once (16-byte loads when the row allows) and scores all HPW
 // heads against it; in the PV phase a lane owns value channels and every
 // value it reads feeds all HPW heads. With one kv head for all query heads
-// (latent caches) the cache is read H / HPW times instead of H times.
+// (latent caches) the cache is read H / HPW times instead of H times. The
+// workgroup has kDecWaves waves, so a context of 1024 keys is one tile per
+// wave: the grid of a decode batch alone rarely fills the chip.
+constexpr int kDecWaves = 16;
+
 template <typename T, int NV, int HPW>
-__global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
+__global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
     T* __restrict__ out, long out_stride,
     const T* __restrict__ q, long q_stride,
     const T* __restrict__ gate, long g_stride,
@@ -639,9 +643,10 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int Dq = (D + 3) & ~3;         // padded so float4 reads stay in a head's row
   float* Qs = smem;                    // [HPW][Dq]
-  float* Ms = Qs + HPW * Dq;           // [4][HPW] max, [4][HPW] sum
-  float* As = Ms + 8 * HPW;            // [4][HPW][DV]
-  for (int idx = tid; idx < HPW * Dq; idx += 256) {
+  constexpr int NW = kDecWaves, NT = 64 * kDecWaves;
+  float* Ms = Qs + HPW * Dq;           // [NW][HPW] max, [NW][HPW] sum
+  float* As = Ms + 2 * NW * HPW;       // [NW][HPW][DV]
+  for (int idx = tid; idx < HPW * Dq; idx += NT) {
     const int hh = idx / Dq, d = idx % Dq;
     Qs[idx] = d < D ? to_f32(q[(long)b * q_stride + (long)(h0 + hh) * D + d]) * scale : 0.f;
   }
@@ -659,7 +664,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
 #pragma unroll
     for (int n = 0; n < NV; ++n) acc[hh][n] = 0.f;
   }
-  for (int kt = lo + w * 64; kt <= i; kt += 4 * 64) {
+  for (int kt = lo + w * 64; kt <= i; kt += NW * 64) {
     const int nk = min(64, i + 1 - kt);
     const int key = kt + lane;
     long base = 0;
@@ -731,7 +736,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
   for (int hh = 0; hh < HPW; ++hh) {
     if (lane == 0) {
       Ms[w * HPW + hh] = m[hh];
-      Ms[(4 + w) * HPW + hh] = l[hh];
+      Ms[(NW + w) * HPW + hh] = l[hh];
     }
 #pragma unroll
     for (int n = 0; n < NV; ++n) {
@@ -740,15 +745,17 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_decode_kernel(
     }
   }
   __syncthreads();
-  for (int idx = tid; idx < HPW * DV; idx += 256) {
+  for (int idx = tid; idx < HPW * DV; idx += NT) {
     const int hh = idx / DV, c = idx % DV;
-    const float mm = fmaxf(fmaxf(Ms[hh], Ms[HPW + hh]), fmaxf(Ms[2 * HPW + hh], Ms[3 * HPW + hh]));
+    float mm = -INFINITY;
+#pragma unroll
+    for (int ww = 0; ww < NW; ++ww) mm = fmaxf(mm, Ms[ww * HPW + hh]);
     float a = 0.f, ll = 0.f;
 #pragma unroll
-    for (int ww = 0; ww < 4; ++ww) {
+    for (int ww = 0; ww < NW; ++ww) {
       const float mw = Ms[ww * HPW + hh];
       const float f = mw > -INFINITY ? expf(mw - mm) : 0.f;
-      ll += Ms[(4 + ww) * HPW + hh] * f;
+      ll += Ms[(NW + ww) * HPW + hh] * f;
       a += As[((long)ww * HPW + hh) * DV + c] * f;
     }
     float gs = 1.f;
