@@ -474,7 +474,7 @@ class KosalornSpec:
         or state."""
         n = len(self.layers)
         a, b, times = self.loop_start, self.loop_stop, self.loop_times
-        if times <= 1 or b <= a:
+        if times == 1 or b <= a:
             return [(i, False) for i in range(n)]
         order = [(i, False) for i in range(a)]
         for p in range(times):

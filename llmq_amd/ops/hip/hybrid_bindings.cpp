@@ -266,7 +266,9 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
     else launch.template operator()<8, 16>();
     return;
   }
-  const size_t lds = sizeof(float) * ((size_t)kAttnKT * (a.D + 1) + (size_t)kAttnKT * a.DV +
+  const bool alias = a.vptr == k_cache.data_ptr();
+  const size_t lds = sizeof(float) * ((size_t)kAttnKT * (a.D + 1) +
+                                      (alias ? 0 : (size_t)kAttnKT * a.DV) +
                                       (size_t)kAttnQT * a.D + (size_t)kAttnQT * kAttnKT);
   const dim3 grid((max_q + kAttnQT - 1) / kAttnQT, a.H, B);
   hy_dispatch(q, "chunk_bias_attn_prefill", [&]<typename T>() {
@@ -298,9 +300,13 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
   TORCH_CHECK(context_lens.numel() == B && block_tables.size(0) == B);
   // query heads per workgroup: as many of one kv head's as divide evenly
   const int per_kv = a.H / a.G;
-  const int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 2 == 0 ? 2 : 1;
-  const size_t lds = sizeof(float) * ((size_t)hpw * ((a.D + 3) & ~3) + 2 * kDecWaves * hpw +
-                                      (size_t)kDecWaves * hpw * a.DV);
+  int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 2 == 0 ? 2 : 1;
+  auto lds_for = [&](int n) {
+    return sizeof(float) * ((size_t)n * ((a.D + 3) & ~3) + 2 * kDecWaves * n +
+                            (size_t)kDecWaves * n * a.DV);
+  };
+  while (hpw > 1 && lds_for(hpw) > 96 * 1024) hpw /= 2;   // wide heads: fewer per workgroup
+  const size_t lds = lds_for(hpw);
   hy_dispatch(q, "paged_attn_decode", [&]<typename T>() {
     dispatch_nv(a.DV, [&]<int NV>() {
       auto launch = [&]<int HPW>() {

@@ -260,9 +260,13 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
   const int pos_last = pos0 + rows - 1;
   const int g = h / (H / G);
   const int DP = D + 1;
+  // values that are the first channels of the key rows are read out of the
+  // K tile: no V tile of their own
+  const bool v_alias = v_cache == k_cache;
+  const int VP = v_alias ? DP : DV;         // row stride of the V tile
   float* Ks = smem;                         // [KT][D+1]
-  float* Vs = Ks + kAttnKT * DP;            // [KT][DV]
-  float* Qs = Vs + kAttnKT * DV;            // [QT][D]
+  float* Vs = v_alias ? Ks : Ks + kAttnKT * DP;            // [KT][DV]
+  float* Qs = Ks + kAttnKT * DP + (v_alias ? 0 : kAttnKT * DV);   // [QT][D]
   float* Ps = Qs + kAttnQT * D;             // [QT][KT]
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
 
@@ -292,7 +296,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
                          key % block_size);
       Ks[jj * DP + d] = to_f32(k_cache[base * D + d]);
     }
-    for (int idx = tid; idx < nk * DV; idx += 256) {
+    for (int idx = tid; idx < (v_alias ? 0 : nk * DV); idx += 256) {
       const int jj = idx / DV, d = idx % DV;
       const int key = kt + jj;
       const long base = (((long)bt[key / block_size] * G + g) * block_size +
@@ -343,7 +347,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
         const float* p0 = Ps + (w * 4) * kAttnKT;
         float a0 = 0.f, a1 = 0.f, a2 = 0.f, a3 = 0.f;
         for (int jj = 0; jj < nk; ++jj) {
-          const float vv = Vs[jj * DV + c];
+          const float vv = Vs[jj * VP + c];
           a0 += p0[jj] * vv;
           a1 += p0[kAttnKT + jj] * vv;
           a2 += p0[2 * kAttnKT + jj] * vv;

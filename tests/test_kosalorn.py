@@ -245,6 +245,10 @@ def test_config_reader_takes_everything_from_config(tmp_path):
     assert [add for _, add in spec.runs()] == [False, False, False, True, False, True, False,
                                                False, False]
     assert [i for i, _ in spec.runs()] == [i for i, _ in oracle.layer_order(cfg)]
+    for loop in ((0, 5, 2), (2, 2, 3), (4, 5, 1), (1, 4, 0)):
+        c2 = make_config(mixed_layers(True), loop=loop)
+        p2 = write_checkpoint(tmp_path / ("m%d%d%d" % loop), c2, make_tensors(c2))
+        assert resolve_spec(p2).runs() == oracle.layer_order(c2), loop
     # every run owns a cache or a state entry
     eng = make_engine(path, ("cpu", "float32"))
     assert len(eng.kv_cache.k) == 9 and len(eng.state_cache.state) == 9
@@ -480,6 +484,8 @@ def test_causal_sees_far_keys_and_page_borders(target, decode):
     (2, 136, 128, 300),
     (1, 256, 192, 70),        # the widest instantiation
     (3, 20, 10, 9),           # not a multiple of 8: the fp32-ALU kernel in bf16 too
+    (8, 288, 256, 40),        # wider than the matrix-core kernel's tiles; 8 heads a group
+    (12, 24, 16, 33),         # 4 heads a group
     (2, 24, 24, 0),           # values = the whole key row, no window
 ])
 def test_window_attention_ops_against_dense(target, H, D, DV, window):
