@@ -305,7 +305,7 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
     return sizeof(float) * ((size_t)n * ((a.D + 3) & ~3) + 2 * kDecWaves * n +
                             (size_t)kDecWaves * n * a.DV);
   };
-  while (hpw > 1 && lds_for(hpw) > 96 * 1024) hpw /= 2;   // wide heads: fewer per workgroup
+  while (hpw > 1 && lds_for(hpw) > 150 * 1024) hpw /= 2;   // wide heads: fewer per workgroup
   const size_t lds = lds_for(hpw);
   hy_dispatch(q, "paged_attn_decode", [&]<typename T>() {
     dispatch_nv(a.DV, [&]<int NV>() {
