@@ -455,7 +455,7 @@ def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q,
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
         _HY.paged_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
-                               q_start, int(max_q), int(span), float(scale), _MASK_BLOCK)
+                               q_start, int(max_q), int(span), float(scale), _MASK_BLOCK, 1)
         return out
     return torch_ref.chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables,
                                              cu_q, q_start, span, scale)
@@ -525,7 +525,7 @@ def window_attn_prefill(q, k_cache, v_cache, dv: int, block_tables, cu_q, q_star
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
         _HY.paged_attn_prefill(out, q, None, k_cache, v_cache, None, block_tables, cu_q, q_start,
-                               int(max_q), int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW)
+                               int(max_q), int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 1)
         return out
     return torch_ref.window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start,
                                          window, scale)
@@ -535,12 +535,37 @@ def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens,
                        scale: float) -> torch.Tensor:
     """The single-token form: query b sits at position context_lens[b]-1."""
     if _use_hybrid(q):
-        out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
+        B, H, D = q.shape
+        out = torch.empty(B, H, dv, dtype=q.dtype, device=q.device)
+        if (q.dtype == torch.bfloat16 and k_cache.shape[1] == 1 and H >= 8 and D % 8 == 0
+                and D <= 256 and q.is_contiguous()):
+            # one kv head for all query heads: the heads of a token become the
+            # rows of one head, all at the token's position, and the step runs
+            # on the matrix-core kernel — every key tile staged once for all
+            # heads instead of once per head group
+            cu = _head_row_offsets(B, H, q.device)
+            _HY.paged_attn_prefill(out.view(B * H, 1, dv), q.view(B * H, 1, D), None, k_cache,
+                                   v_cache, None, block_tables, cu, context_lens - 1, H,
+                                   int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 0)
+            return out
         _HY.paged_attn_decode(out, q, None, k_cache, v_cache, None, block_tables, context_lens,
                               int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW)
         return out
     return torch_ref.window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens,
                                         window, scale)
+
+
+_HEAD_ROWS = {}
+
+
+def _head_row_offsets(B: int, H: int, device) -> torch.Tensor:
+    """[0, H, 2H, ..., B*H] int32 on the device, made once per (B, H)."""
+    key = (B, H, str(device))
+    t = _HEAD_ROWS.get(key)
+    if t is None:
+        t = torch.arange(B + 1, dtype=torch.int32, device=device) * H
+        _HEAD_ROWS[key] = t
+    return t
 
 
 def latent_rope_pack(q, q_lat, ckr, c_w, inv_freq, positions, k_cache, slots, dim: int,

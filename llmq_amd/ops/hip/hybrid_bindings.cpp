@@ -226,8 +226,9 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                         at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
                         const std::optional<at::Tensor>& bias, at::Tensor block_tables,
                         at::Tensor cu_q, at::Tensor q_start, int64_t max_q, int64_t span,
-                        double scale, int64_t mask_mode) {
+                        double scale, int64_t mask_mode, int64_t pos_stride) {
   if (q.size(0) == 0) return;
+  TORCH_CHECK(pos_stride == 0 || pos_stride == 1, "pos_stride is 0 (rows share a position) or 1");
   const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode);
   HY_I32(cu_q); HY_I32(q_start);
   const int B = q_start.numel();
@@ -238,7 +239,10 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
     const char* e = getenv("LLMQ_HYBRID_ATTN_VALU");
     return e && e[0] == '1';
   }();
-  if (q.scalar_type() == at::kBFloat16 && !force_valu && a.D % 8 == 0 && a.D <= 256 &&
+  TORCH_CHECK(pos_stride == 1 || (q.scalar_type() == at::kBFloat16 && a.D % 8 == 0 && a.D <= 256 &&
+                                  q.stride(0) % 8 == 0 && !gate.has_value()),
+              "rows that share a position run on the matrix-core kernel only");
+  if (q.scalar_type() == at::kBFloat16 && (!force_valu || pos_stride == 0) && a.D % 8 == 0 && a.D <= 256 &&
       q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
     const int ksn = (a.D + 31) / 32, dtn = (a.DV + 15) / 16;
     const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H, B);
@@ -259,7 +263,7 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          reinterpret_cast<const bf*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale, a.v_row, (int)mask_mode);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)pos_stride);
     };
     if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
     else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
@@ -635,7 +639,7 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("sandwich_norm_res32(Tensor(a!) x, Tensor(b!) residual, Tensor w_post, Tensor w_pre, float eps, float offset) -> ()");
   m.def("act_and_mul(Tensor(a!) out, Tensor input, bool gelu) -> ()");
   m.def("qknorm_vmix_cache(Tensor(a!) q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, Tensor? v_first, float lam, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slots, float eps) -> ()");
-  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode) -> ()");
+  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode, int pos_stride) -> ()");
   m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode) -> ()");
   m.def("gla_recurrence(Tensor(a!) o, Tensor q, Tensor? k, Tensor v, Tensor z, Tensor z_bias, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float tau, Tensor? lower, bool q_silu, float q_scale) -> ()");
   m.def("gla_out_norm_gate(Tensor(a!) out, Tensor o, Tensor weight, Tensor? gate, float eps) -> ()");

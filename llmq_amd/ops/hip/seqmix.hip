@@ -405,7 +405,12 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode) {
+    int v_row, int mask_mode, int ps) {
+  // ps = 1: row r of a sequence sits at position q_start + r (a prompt
+  // portion). ps = 0: all rows of a sequence sit at q_start — the rows are the
+  // query HEADS of one new token that share one kv head, laid out as rows of
+  // a single head, so a decode step over a latent cache runs on the matrix
+  // cores with every key tile staged once for all heads.
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr int VG = DT / 2;             // 32-channel groups of V per thread
   const int b = blockIdx.z, h = blockIdx.y;
@@ -414,8 +419,8 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   const int r0 = blockIdx.x * kMfmaQT;
   if (r0 >= nq) return;
   const int rows = min(kMfmaQT, nq - r0);
-  const int pos0 = q_start[b] + r0;
-  const int pos_last = pos0 + rows - 1;
+  const int pos0 = q_start[b] + r0 * ps;
+  const int pos_last = pos0 + (rows - 1) * ps;
   const int g = h / (H / G);
   const int ksn = (D + 31) / 32, dtn = (DV + 15) / 16;
   const bool v_alias = v_cache == k_cache;             // values = prefix of the key rows
@@ -443,16 +448,16 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 #pragma unroll
   for (int reg = 0; reg < 4; ++reg) {
     const int r = w * 16 + kgrp * 4 + reg;
-    irow[reg] = r < rows ? pos0 + r : -1;       // -1: no key satisfies key <= irow
-    lorow[reg] = r < rows ? mask_first_key(pos0 + r, span, mask_mode) : 0;
+    irow[reg] = r < rows ? pos0 + r * ps : -1;  // -1: no key satisfies key <= irow
+    lorow[reg] = r < rows ? mask_first_key(pos0 + r * ps, span, mask_mode) : 0;
     m[reg] = -INFINITY;
     l[reg] = 0.f;
   }
   sm_f32x4 o[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) o[dt] = sm_f32x4{0.f, 0.f, 0.f, 0.f};
-  const int wave_first = pos0 + w * 16;
-  const int wave_last = min(pos_last, wave_first + 15);
+  const int wave_first = pos0 + w * 16 * ps;
+  const int wave_last = min(pos_last, wave_first + 15 * ps);
   const int wave_lo = mask_first_key(wave_first, span, mask_mode);
   const bool wave_rows = w * 16 < rows;
   const int* bt = block_tables + (long)b * bt_stride;
@@ -538,7 +543,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 #pragma unroll
       for (int reg = 0; reg < 4; ++reg) {
         float sv[4], tmax = -INFINITY;
-        const float* brow = Bs + (w * 16 + kgrp * 4 + reg) + 63 - col;
+        const float* brow = Bs + (w * 16 + kgrp * 4 + reg) * ps + 63 - col;
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
           const int key = kt + ct * 16 + col;

@@ -409,8 +409,9 @@ def test_long_decode_across_windows_and_pages(mixed_model, target):
 
 # ------------------------------------------ edges made visible by design --
 
-def _needle_case(device, dtype, window, key_pos, query_pos, decode, block_size=16, DV=8, D=12):
-    """One latent cache, two heads; every key scores 0 but the needle, whose
+def _needle_case(device, dtype, window, key_pos, query_pos, decode, block_size=16, DV=8, D=16,
+                 heads=2):
+    """One latent cache, two heads (or more: many heads take another kernel); every key scores 0 but the needle, whose
     first channel is 40: the output is the needle's value prefix iff the
     query may see it. Values are the first DV channels of the key rows."""
     from llmq_amd import ops
@@ -427,16 +428,17 @@ def _needle_case(device, dtype, window, key_pos, query_pos, decode, block_size=1
     kc[b, 0, o, 1] = -3.0
     kc, table = kc.to(device), table.to(device)
     if decode:
-        q = torch.zeros(1, 2, D, dtype=dtype, device=device)
+        q = torch.zeros(1, heads, D, dtype=dtype, device=device)
         q[0, :, 0] = 1.0
         out = ops.window_attn_decode(
             q, kc, None, DV, table, torch.tensor([n], dtype=torch.int32, device=device),
             window, 1.0)
-        assert out.shape == (1, 2, DV)
+        assert out.shape == (1, heads, DV)
+        assert torch.equal(out[0, 1], out[0, heads - 1])
         return float(out[0, 1, 1])
     start = max(0, query_pos - 4)            # a portion whose last row is the query
     rows = query_pos - start + 1
-    q = torch.zeros(rows, 2, D, dtype=dtype, device=device)
+    q = torch.zeros(rows, heads, D, dtype=dtype, device=device)
     q[:, :, 0] = 1.0
     out = ops.window_attn_prefill(
         q, kc, None, DV, table, torch.tensor([0, rows], dtype=torch.int32, device=device),
@@ -455,11 +457,15 @@ def test_window_edges_with_a_needle(target, decode):
             oldest = max(0, query_pos - window + 1)      # the oldest key still seen
             seen = _needle_case(device, dtype, window, oldest, query_pos, decode)
             assert seen < -2.9, (window, query_pos, seen)
+            many = _needle_case(device, dtype, window, oldest, query_pos, decode, heads=19)
+            assert many < -2.9, (window, query_pos, many)
             newest = _needle_case(device, dtype, window, query_pos, query_pos, decode)
             assert newest < -2.9, (window, query_pos, newest)
             if oldest > 0:                                # one further back is outside
                 unseen = _needle_case(device, dtype, window, oldest - 1, query_pos, decode)
                 assert unseen > 0.99, (window, query_pos, unseen)
+                many = _needle_case(device, dtype, window, oldest - 1, query_pos, decode, heads=19)
+                assert many > 0.99, (window, query_pos, many)
                 assert _needle_case(device, dtype, window, 0, query_pos, decode) > 0.99
 
 
@@ -486,6 +492,8 @@ def test_causal_sees_far_keys_and_page_borders(target, decode):
     (3, 20, 10, 9),           # not a multiple of 8: the fp32-ALU kernel in bf16 too
     (8, 288, 256, 40),        # wider than the matrix-core kernel's tiles; 8 heads a group
     (12, 24, 16, 33),         # 4 heads a group
+    (16, 64, 48, 70),         # many heads on one latent: single tokens on the matrix cores
+    (70, 136, 128, 0),        # more heads than one workgroup's rows
     (2, 24, 24, 0),           # values = the whole key row, no window
 ])
 def test_window_attention_ops_against_dense(target, H, D, DV, window):
