@@ -245,7 +245,19 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
   if (q.scalar_type() == at::kBFloat16 && (!force_valu || pos_stride == 0) && a.D % 8 == 0 && a.D <= 256 &&
       q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
     const int ksn = (a.D + 31) / 32, dtn = (a.DV + 15) / 16;
-    const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H, B);
+    // rows that share a position (single tokens): a sequence is one
+    // workgroup per 64 heads, so its keys are split over several until the
+    // grid has about two workgroups per CU; the partials are merged below
+    int n_split = 1;
+    at::Tensor part;
+    if (pos_stride == 0) {
+      const long wgs = (long)((max_q + kMfmaQT - 1) / kMfmaQT) * a.H * B;
+      const long max_tiles = std::max<long>(1, block_tables.size(1) * (long)a.bs / kMfmaKT);
+      n_split = (int)std::min<long>(std::min<long>(8, max_tiles), std::max<long>(1, 512 / wgs));
+      if (n_split > 1)
+        part = at::empty({q.size(0), a.H, n_split, a.DV + 2}, q.options().dtype(at::kFloat));
+    }
+    const dim3 grid((max_q + kMfmaQT - 1) / kMfmaQT, a.H * n_split, B);
     using bf = __hip_bfloat16;
     auto launch = [&]<int KS, int DT>() {
       // K tile, V^T tile (the channel tiles in use), P hi/lo per wave, bias slice
@@ -263,11 +275,18 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          reinterpret_cast<const bf*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)pos_stride);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)pos_stride,
+                         n_split, n_split > 1 ? part.data_ptr<float>() : nullptr);
     };
     if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
     else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
     else launch.template operator()<8, 16>();
+    if (n_split > 1) {
+      const long pairs = q.size(0) * (long)a.H;
+      hipLaunchKernelGGL(attn_merge_splits_kernel, dim3((pairs + 3) / 4), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<bf*>(out.data_ptr()), out.stride(0),
+                         part.data_ptr<float>(), pairs, a.H, a.DV, n_split);
+    }
     return;
   }
   const bool alias = a.vptr == k_cache.data_ptr();

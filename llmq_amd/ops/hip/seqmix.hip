@@ -405,7 +405,11 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode, int ps) {
+    int v_row, int mask_mode, int ps, int n_split, float* __restrict__ part) {
+  // n_split > 1: the grid's y dimension carries (key split, head); a
+  // workgroup walks only its share of the key tiles and writes its
+  // unnormalised output, running maximum and sum to `part`
+  // [row, head, split, DV + 2] for attn_merge_splits_kernel.
   // ps = 1: row r of a sequence sits at position q_start + r (a prompt
   // portion). ps = 0: all rows of a sequence sit at q_start — the rows are the
   // query HEADS of one new token that share one kv head, laid out as rows of
@@ -413,7 +417,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   // cores with every key tile staged once for all heads.
   extern __shared__ __align__(16) unsigned char smem_raw[];
   constexpr int VG = DT / 2;             // 32-channel groups of V per thread
-  const int b = blockIdx.z, h = blockIdx.y;
+  const int b = blockIdx.z, h = blockIdx.y % H, sp = blockIdx.y / H;
   const int row0 = cu_q[b];
   const int nq = cu_q[b + 1] - row0;
   const int r0 = blockIdx.x * kMfmaQT;
@@ -500,9 +504,16 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       vreg[i] = e;
     }
   };
-  const int kt0 = mask_first_key(pos0, span, mask_mode);
-  fetch(kt0);
-  for (int kt = kt0; kt <= pos_last; kt += kMfmaKT) {
+  int kt0 = mask_first_key(pos0, span, mask_mode);
+  int key_end = pos_last;                // last key this workgroup visits
+  if (n_split > 1) {
+    const int tiles = (pos_last - kt0) / kMfmaKT + 1;
+    const int chunk = (tiles + n_split - 1) / n_split;
+    kt0 += sp * chunk * kMfmaKT;
+    key_end = min(pos_last, kt0 + chunk * kMfmaKT - 1);
+  }
+  if (kt0 <= key_end) fetch(kt0);
+  for (int kt = kt0; kt <= key_end; kt += kMfmaKT) {
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
@@ -524,7 +535,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       Bs[tid] = (bias_h && d >= 0 && d < bias_len) ? bias_h[d] : 0.f;
     }
     __syncthreads();
-    if (kt + kMfmaKT <= pos_last) fetch(kt + kMfmaKT);
+    if (kt + kMfmaKT <= key_end) fetch(kt + kMfmaKT);
     const bool active = wave_rows && kt <= wave_last && kt + kMfmaKT - 1 >= wave_lo;
     if (active) {
       sm_f32x4 s[4];
@@ -610,6 +621,19 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int r = w * 16 + kgrp * 4 + reg;
     if (r >= rows) continue;
     const long trow = row0 + r0 + r;
+    if (n_split > 1) {
+      float* pr = part + ((trow * H + h) * n_split + sp) * (long)(DV + 2);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        const int c = dt * 16 + col;
+        if (dt < dtn && c < DV) pr[c] = o[dt][reg];
+      }
+      if (col == 0) {
+        pr[DV] = m[reg];
+        pr[DV + 1] = ll;
+      }
+      continue;
+    }
     float gs = 1.f;
     if (gate) gs = 1.0f / (1.0f + expf(-__bfloat162float(gate[trow * g_stride + h])));
     const float inv = gs / ll;
@@ -619,6 +643,35 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       if (dt < dtn && c < DV)
         out[trow * out_stride + (long)h * DV + c] = __float2bfloat16(o[dt][reg] * inv);
     }
+  }
+}
+
+// Merge of key splits: out[row, head] = sum_s o_s e^(m_s - M) / sum_s l_s e^(m_s - M),
+// M = max_s m_s; a split that saw no key has m = -inf and counts nothing.
+// One wave per (row, head), lanes over value channels.
+__global__ __launch_bounds__(256) void attn_merge_splits_kernel(
+    __hip_bfloat16* __restrict__ out, long out_stride, const float* __restrict__ part,
+    long pairs, int H, int DV, int n_split) {
+  const long pair = blockIdx.x * 4L + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const float* pp = part + pair * n_split * (long)(DV + 2);
+  float M = -INFINITY;
+  for (int sidx = 0; sidx < n_split; ++sidx) M = fmaxf(M, pp[sidx * (DV + 2) + DV]);
+  float L = 0.f;
+  for (int sidx = 0; sidx < n_split; ++sidx) {
+    const float ms = pp[sidx * (DV + 2) + DV];
+    if (ms > -INFINITY) L += pp[sidx * (DV + 2) + DV + 1] * expf(ms - M);
+  }
+  const long row = pair / H;
+  const int h = (int)(pair % H);
+  for (int c = lane; c < DV; c += 64) {
+    float a = 0.f;
+    for (int sidx = 0; sidx < n_split; ++sidx) {
+      const float ms = pp[sidx * (DV + 2) + DV];
+      if (ms > -INFINITY) a += pp[sidx * (DV + 2) + c] * expf(ms - M);
+    }
+    out[row * out_stride + (long)h * DV + c] = __float2bfloat16(a / L);
   }
 }
 
