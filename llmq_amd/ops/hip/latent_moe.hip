@@ -3,7 +3,7 @@
 // parallel residual join, the token-indexed side gate, the sigmoid top-k
 // router and the matrix-vector form of an expert mixture.
 //
-// Numerics contract as in seqmix.hip: activations arrive in the model dtype T
+// Numerics as in seqmix.hip: activations arrive in the model dtype T
 // (bf16 or fp32); angles, norms, gates, router scores and the residual are
 // fp32 in registers and rounded to T once, on store.
 

@@ -296,6 +296,25 @@ def test_mechanism_alone(tmp_path, target, layers, side, loop):
     assert_close(got, want, target, "logits")
 
 
+@pytest.mark.parametrize("target", DEVICES)
+def test_sizes_that_fit_no_vector_width(tmp_path, target):
+    """Width, vocabulary, ranks and head sizes that are multiples of nothing:
+    every kernel takes its scalar path, GEMM operands are unaligned."""
+    layers = [
+        latent(heads=3, dim=5, rot_dim=6, vdim=7, kv_rank=11, q_rank=9, window=13, mlp="dense"),
+        hgrn2(heads=3, dim=7, vdim=9, mlp=(3, 3)),
+        latent2(heads=9, dim=6, rot_dim=2, vdim=5, kv_rank=14, mlp=None),
+    ]
+    cfg = make_config(layers, width=50, vocab=101, side=5, loop=(0, 2, 2))
+    tensors = make_tensors(cfg, seed=3)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    toks = tokens_for(60, cfg["vocab"], 6)
+    want = oracle.forward(cfg, tensors, toks)
+    eng = make_engine(path, target)
+    assert_close(replay(eng, "a", toks, [60]), want, target, "whole")
+    assert_close(replay(eng, "b", toks, [7, 2, 30, 1, 1, 19]), want, target, "cut")
+
+
 @pytest.mark.parametrize("target", DEVICES[:2])
 @pytest.mark.parametrize("experts,top", [(5, 1), (5, 2), (7, 3), (2, 1)])
 def test_expert_choice_in_the_model(tmp_path, target, experts, top):
