@@ -517,7 +517,8 @@ def kosalorn_spec_from_config(cfg: dict, name: str) -> KosalornSpec:
             mask = mc.get("mask")
             mixer = LatentAttnSpec(
                 heads=int(mc["heads"]), dim=int(mc["dim"]), rot_dim=int(mc["rot_dim"]),
-                vdim=int(mc["vdim"]), kv_rank=int(mc["kv_rank"]), scale=float(mc["scale"]),
+                vdim=int(mc["vdim"]), kv_rank=int(mc["kv_rank"]),
+                scale=float(mc.get("scale", (int(mc["dim"]) + int(mc["rot_dim"])) ** -0.5)),
                 rot=RotarySpec(base=float(rot["base"]), dims=int(rot["dims"]),
                                layout="half" if kind == "latent_attention" else "interleaved"),
                 q_rank=int(mc.get("q_rank", 0)) if kind == "latent_attention" else 0,

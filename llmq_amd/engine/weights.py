@@ -254,7 +254,7 @@ def load_kosalorn_weights(model, path: Path) -> None:
             copy_(t["side_norm"], get(p + "side.norm"))
     unused = sorted(set(tensors) - used)
     if unused:
-        raise ValueError(f"checkpoint tensors the model does not know: {unused[:8]}")
+        logger.warning("checkpoint tensors this configuration does not use: %s", unused[:8])
     model.finalize()
     logger.info("loaded %d tensors from %s", len(tensors), path)
 

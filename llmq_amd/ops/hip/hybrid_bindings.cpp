@@ -196,7 +196,7 @@ AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optio
   }
   TORCH_CHECK(out.size(0) == q.size(0) && out.size(1) == a.H);
   TORCH_CHECK(a.H % a.G == 0, "heads must be a multiple of kv heads");
-  TORCH_CHECK(a.DV >= 1 && a.DV <= 256, "value size above 256 is not supported");
+  TORCH_CHECK(a.DV >= 1 && a.DV <= 512, "value size above 512 is not supported");
   TORCH_CHECK(span >= 1);
   if (bias.has_value()) {
     TORCH_CHECK(bias->scalar_type() == at::kFloat && bias->is_contiguous() && bias->dim() == 2 &&
@@ -219,7 +219,8 @@ template <typename F>
 void dispatch_nv(int DV, F&& f) {
   if (DV <= 64) f.template operator()<1>();
   else if (DV <= 128) f.template operator()<2>();
-  else f.template operator()<4>();
+  else if (DV <= 256) f.template operator()<4>();
+  else f.template operator()<8>();
 }
 
 void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,

@@ -510,6 +510,7 @@ def test_causal_sees_far_keys_and_page_borders(target, decode):
     (1, 256, 192, 70),        # the widest instantiation
     (3, 20, 10, 9),           # not a multiple of 8: the fp32-ALU kernel in bf16 too
     (8, 288, 256, 40),        # wider than the matrix-core kernel's tiles; 8 heads a group
+    (2, 320, 300, 50),        # values wider than 256
     (12, 24, 16, 33),         # 4 heads a group
     (16, 64, 48, 70),         # many heads on one latent: single tokens on the matrix cores
     (70, 136, 128, 0),        # more heads than one workgroup's rows
